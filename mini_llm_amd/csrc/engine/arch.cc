@@ -19,6 +19,7 @@ void register_builtin_architectures() {
     static std::once_flag once;
     std::call_once(once, [] {
         register_gpt2();
+        register_kugulorn();
         if (const char* env = std::getenv("MINI_LLM_PLUGINS")) {
             std::stringstream ss(env);
             for (std::string path; std::getline(ss, path, ':');)
@@ -68,6 +69,10 @@ const Architecture& architecture_of(const Json& config) {
     std::string name;
     if (const Json* a = config.find("architectures"))
         if (a->is_array() && !a->array().empty() && a->array()[0].is_string()) name = a->array()[0].string();
+    if (name.empty() || !archs().count(name)) {
+        if (const Json* a = config.find("architecture"))
+            if (a->is_string() && archs().count(a->string())) name = a->string();
+    }
     if (name.empty() || !archs().count(name)) {
         if (const Json* t = config.find("model_type"))
             if (t->is_string() && by_model_type().count(t->string())) name = by_model_type()[t->string()];

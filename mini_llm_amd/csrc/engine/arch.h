@@ -48,10 +48,12 @@ struct Architecture {
 // and `out.eos_token_id`; the caches' needs are read off the model afterwards.
 void register_architecture(const Architecture& a, const std::string& model_type = "");
 void register_gpt2();              // gpt2.cc
+void register_kugulorn();          // kugulorn.cc
 // Loads a shared library whose initialisers register parts and architectures (dlopen; stays loaded).
 // Also called for every path in the environment variable MINI_LLM_PLUGINS (colon-separated), once.
 void load_plugin(const std::string& path);
-// by config.json: architectures[0], else model_type; unknown -> ConfigError listing the registered names
+// by config.json: architectures[0], else the string "architecture", else model_type; unknown -> ConfigError
+// listing the registered names
 const Architecture& architecture_of(const Json& config);
 std::vector<std::string> registered_architectures();
 

@@ -34,13 +34,13 @@ CacheStorage::CacheStorage(const std::vector<CacheNeed>& needs, int page_size, i
 
 void CacheStorage::allocate(const std::vector<CacheNeed>& needs, int n_pages, int n_state_slots) {
     const int page_size = page_size_, dtype = dtype_;
-    struct Key { int hkv, hd, window; bool operator==(const Key& o) const { return hkv == o.hkv && hd == o.hd && window == o.window; } };
+    struct Key { int hkv, hd, vd, window; bool operator==(const Key& o) const { return hkv == o.hkv && hd == o.hd && vd == o.vd && window == o.window; } };
     std::vector<Key> keys;
     std::vector<std::vector<int>> members;
     std::vector<int> group_of(needs.size(), -1);
     for (size_t c = 0; c < needs.size(); ++c) {
         if (needs[c].kind != 1) continue;
-        const Key k{needs[c].n_kv_heads, needs[c].head_dim, needs[c].window};
+        const Key k{needs[c].n_kv_heads, needs[c].head_dim, needs[c].value_dim < 0 ? needs[c].head_dim : needs[c].value_dim, needs[c].window};
         size_t g = 0;
         while (g < keys.size() && !(keys[g] == k)) ++g;
         if (g == keys.size()) { keys.push_back(k); members.emplace_back(); }
@@ -56,8 +56,9 @@ void CacheStorage::allocate(const std::vector<CacheNeed>& needs, int n_pages, in
         gs.window = keys[g].window;
         group_specs_.push_back(gs);
         const int64_t rows = static_cast<int64_t>(n_pages) * page_size, kv_dim = static_cast<int64_t>(keys[g].hkv) * keys[g].hd;
-        const size_t one = static_cast<size_t>(rows) * kv_dim * esz;
-        const size_t bytes = one * 2 * members[g].size();
+        const int64_t v_dim = static_cast<int64_t>(keys[g].hkv) * keys[g].vd;         // 0: key rows only
+        const size_t k_bytes = static_cast<size_t>(rows) * kv_dim * esz, v_bytes = static_cast<size_t>(rows) * v_dim * esz;
+        const size_t bytes = (k_bytes + v_bytes) * members[g].size();
         void* pool = nullptr;
         HIP_OK(hipMalloc(&pool, std::max<size_t>(bytes, 16)));
         allocations_.push_back(pool);
@@ -66,12 +67,12 @@ void CacheStorage::allocate(const std::vector<CacheNeed>& needs, int n_pages, in
         for (size_t j = 0; j < members[g].size(); ++j) {
             CacheView& v = views_[members[g][j]];
             v.kind = 1;
-            v.k_pages = Tensor2(static_cast<char*>(pool) + (2 * j) * one, dtype, rows, kv_dim);
-            v.v_pages = Tensor2(static_cast<char*>(pool) + (2 * j + 1) * one, dtype, rows, kv_dim);
+            v.k_pages = Tensor2(static_cast<char*>(pool) + j * (k_bytes + v_bytes), dtype, rows, kv_dim);
+            v.v_pages = v_dim > 0 ? Tensor2(static_cast<char*>(pool) + j * (k_bytes + v_bytes) + k_bytes, dtype, rows, v_dim) : Tensor2();
             v.group = static_cast<int>(g);
             v.page_size = page_size;
             v.window = keys[g].window;
-            bytes_per_token_ += 2 * static_cast<size_t>(kv_dim) * esz;
+            bytes_per_token_ += static_cast<size_t>(kv_dim + v_dim) * esz;
         }
     }
     for (size_t c = 0; c < needs.size(); ++c) {
@@ -111,7 +112,7 @@ static int pages_for_memory_fraction(const std::vector<CacheNeed>& needs, int dt
     if (fraction > 1.0) throw EngineError("kv_memory_fraction must be at most 1");
     size_t per_token = 0;
     for (const CacheNeed& n : needs)
-        if (n.kind == 1) per_token += 2 * static_cast<size_t>(n.n_kv_heads) * n.head_dim * dtype_size(dtype);
+        if (n.kind == 1) per_token += static_cast<size_t>(n.n_kv_heads) * (n.head_dim + (n.value_dim < 0 ? n.head_dim : n.value_dim)) * dtype_size(dtype);
     if (per_token == 0) return 1;
     size_t free_bytes = 0, total_bytes = 0;
     HIP_OK(hipMemGetInfo(&free_bytes, &total_bytes));

@@ -58,6 +58,36 @@ int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const vo
                                 int head_dim, int page_size, float scale, int window, void* out, int out_stride,
                                 hipStream_t stream);
 
+// norm_gate.hip
+int mllm_rmsnorm(const float* x, int ldx, const int* rows, const float* w, const float* gate, int ldg, void* y, int ldy,
+                 int n, int D, int groups, float eps, int out_dtype, hipStream_t stream);
+int mllm_rmsnorm_add(float* y, const float* w, const float* scale, float mult, float eps, float* x, int n, int D,
+                     int clear, hipStream_t stream);
+int mllm_glu_clamped(const void* gate, int ldg, const void* up, int ldu, void* out, int ldo, int T, int F, float limit,
+                     float alpha, int dtype, hipStream_t stream);
+int mllm_fill_zero(void* p, size_t bytes, hipStream_t stream);
+
+// ssm.hip
+int mllm_conv_silu(const float* proj, int ld, int col0, int C, const float* w, const float* bias, int taps,
+                   const int* token_seq, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
+                   float* out, int ldo, int T, int B, int write, hipStream_t stream);
+int mllm_ssm_scan(const float* xbc, int ldx, const float* raw_dt, int ldd, const float* dt_bias, const float* A_log,
+                  const float* Dskip, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
+                  size_t scan_offset, float* y, int ldy, int B, int H, int P, int N, int G, int write,
+                  hipStream_t stream);
+
+// latent_attention.hip
+int mllm_latent_prepare(const float* dq, int ld_dq, int Rq, const float* wq, void* cq, int ld_cq, const float* dkv, int ld_dkv,
+                        int R, int Dr, const float* wkv, void* pages, const int* slots, const int* positions, int T, float eps,
+                        double base, int rot_dims, int dtype, hipStream_t stream);
+int mllm_latent_absorb(const void* q, int ldq, const void* w_uk, int ldw, void* qa, int ldqa, const int* positions, int T, int H,
+                       int Dn, int Dr, int R, double base, int rot_dims, int dtype, hipStream_t stream);
+int mllm_latent_attention(const void* qa, int ldqa, const void* pages, const int* block_tables, int max_blocks,
+                          const int* token_seq, const int* positions, int T, int H, int R, int Dr, int page_size, float scale,
+                          int window, void* o_lat, int ldo, int dtype, hipStream_t stream);
+int mllm_latent_expand(const void* o_lat, int ldo, const void* w_uv, int ldw, void* out, int ldout, int T, int H, int Dv, int R,
+                       int dtype, hipStream_t stream);
+
 // sampling.hip
 int mllm_argmax_chunks(int V);
 int mllm_argmax_mirrored(const float* logits, int ld, int n, int V, int* out, int* mirror, float* part_val, int* part_idx,

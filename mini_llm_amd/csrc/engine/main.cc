@@ -10,7 +10,7 @@
 //       random weights of that size.
 //   mini-llm make-model (--preset NAME | --config FILE) --seed S --out DIR [--weights-dtype bfloat16|float32]
 //       Writes a model folder with random weights.
-//   mini-llm replay --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--page-size P]
+//   mini-llm replay --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--page-size P] [--max-requests R]
 //       Trace replay: one JSON object a line on standard input
 //       ({"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}), logits of
 //       the wanted places to OUT/<step>.f32, "done <step>" after every step. It samples nothing.
@@ -249,7 +249,7 @@ int cmd_replay(int argc, char** argv) {
     std::fprintf(stderr, "[replay] loading %s as %s ...\n", a.get("model").c_str(), a.get("dtype").c_str());
     std::unique_ptr<LoadedModel> model = load_model(a.get("model"), dtype_of(a.get("dtype")));
     const int n_pages = static_cast<int>((a.integer("max-tokens", 0) + page - 1) / page);
-    ModelRunner runner(*model, page, n_pages, static_cast<int>(a.integer("max-requests", 16)));
+    ModelRunner runner(*model, page, n_pages, static_cast<int>(a.integer("max-requests", 4)));
     const std::string out_dir = a.get("out");
     for (size_t at = 1; at <= out_dir.size(); ++at)      // the folder and the folders above it
         if (at == out_dir.size() || out_dir[at] == '/') ::mkdir(out_dir.substr(0, at).c_str(), 0755);
@@ -332,7 +332,7 @@ int main(int argc, char** argv) {
                  "  every command: [--plugin LIB.so]...  shared libraries that register further parts and architectures\n"
                  "             (also: the paths in the environment variable MINI_LLM_PLUGINS, separated by colons)\n"
                  "  make-model (--preset NAME | --config FILE) --seed S --out DIR [--weights-dtype bfloat16|float32]\n"
-                 "  replay     --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--page-size 16]\n"
+                 "  replay     --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--page-size 16] [--max-requests 4]\n"
                  "  check      --model DIR     (configuration and tensors against the architecture; needs no GPU)\n");
     return cmd.empty() || cmd == "--help" || cmd == "-h" ? (cmd.empty() ? 1 : 0) : 1;
 }

@@ -149,6 +149,62 @@ void ln_linear(const Tensor2& x, const float* gamma, const float* beta, float ep
 // Causal attention of the step's queries over the pages. Returns true and fills *splits when the result is
 // left unmerged (only with may_split); otherwise `out` holds it.
 bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_t stream);
+
+// -- RMS norms, gated activation ---------------------------------------------------------------------
+// out[i, :] = x[rows ? rows[i] : i, :] / sqrt(mean(.^2) + eps) * weight, the columns in `groups` equal parts
+// that are normed one by one; with `gate` (fp32, x's shape) the input is x * silu(gate) (the gate comes
+// before the norm). x fp32 (any row stride), out in its own dtype.
+void rmsnorm(const Tensor2& x, const float* weight, float eps, int groups, const Tensor2* gate, const Tensor2& out,
+             const int* rows, hipStream_t stream);
+// x += mult * scale * (y / sqrt(mean(y^2) + eps) * weight), row by row (scale: per column, or null);
+// `clear`: y is zero afterwards.
+void rmsnorm_add(const Tensor2& y, const float* weight, const float* scale, float mult, float eps, const Tensor2& x,
+                 bool clear, hipStream_t stream);
+// out = g sigmoid(alpha g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit)
+void glu_clamped(const Tensor2& gate, const Tensor2& up, float limit, float alpha, const Tensor2& out, hipStream_t stream);
+void fill_zero(const Tensor2& x, hipStream_t stream);          // contiguous fp32, by a kernel
+
+// -- state-space mixer -------------------------------------------------------------------------------
+// A step's sequences with per-request state slots ([n_slots, slot_floats] fp32).
+struct StateArgs {
+    const int* token_seq = nullptr;    // [T]
+    const int* cu_q = nullptr;         // [B + 1]
+    const int* state_slots = nullptr;  // [B], < 0: padding
+    int n_seqs = 0;
+    float* state = nullptr;
+    size_t slot_floats = 0;
+    int n_slots = 0;
+    bool write = true;
+};
+// out[t, :] = silu(conv(columns [col0, col0 + C) of proj)), causal per sequence over `taps` inputs, the inputs
+// before a portion taken from the slot's first (taps - 1) * C floats, which are brought up to date afterwards.
+void conv_silu(const Tensor2& proj, int col0, const Tensor2& weight, const float* bias, const StateArgs& st,
+               const Tensor2& out, hipStream_t stream);
+// The Mamba-2 scan (kernels/ssm.hip) over xbc [T, H*P + 2*G*N] and the raw step sizes (columns dt_col.. of
+// proj), state at `scan_offset` floats into the slot; y [T, H*P] fp32.
+void ssm_scan(const Tensor2& xbc, const Tensor2& proj, int dt_col, const float* dt_bias, const float* A_log,
+              const float* skip, const StateArgs& st, size_t scan_offset, int H, int P, int N, int G, const Tensor2& y,
+              hipStream_t stream);
+
+// -- latent attention --------------------------------------------------------------------------------
+struct LatentShape {
+    int n_heads = 0, plain_dim = 0, rot_dim = 0, value_dim = 0, kv_rank = 0, q_rank = 0, rot_dims = 0;
+    double rot_base = 10000.0;
+    float eps = 1e-6f;
+};
+// cq = rmsnorm(dq) * wq; with dkv: page row slots[t] = [rmsnorm(dkv[:, :kv_rank]) * wkv | turned rest]
+void latent_prepare(const Tensor2& dq, const float* wq, const Tensor2& cq, const Tensor2* dkv, const float* wkv,
+                    const Tensor2* pages, const int* slots, const int* positions, const LatentShape& sh, hipStream_t stream);
+// qa[t, h] = [W_uk_h^T q_plain[t, h] | turned q_rot[t, h]]
+void latent_absorb(const Tensor2& q, const Tensor2& w_uk, const Tensor2& qa, const int* positions, const LatentShape& sh,
+                   hipStream_t stream);
+// o_lat[t, h] = sum_j softmax_j(scale * qa[t, h] . row_j) row_j[:kv_rank] over the visible rows of the pages
+void latent_attention(const Tensor2& qa, const Tensor2& pages, int page_size, const int* block_tables, int max_blocks,
+                      const int* token_seq, const int* positions, float scale, int window, const LatentShape& sh,
+                      const Tensor2& o_lat, hipStream_t stream);
+// out[t, h*value_dim + e] = sum_r w_uv[h*value_dim + e, r] * o_lat[t, h, r]
+void latent_expand(const Tensor2& o_lat, const Tensor2& w_uv, const Tensor2& out, const LatentShape& sh, hipStream_t stream);
+
 // `mirror` (optional): a second place for the chosen tokens, which may be pinned host memory (the kernel that
 // chooses writes it: no copy has to be launched for the host to read them).
 void argmax(const Tensor2& logits, int* out, hipStream_t stream, int* mirror = nullptr);

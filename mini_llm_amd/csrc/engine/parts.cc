@@ -110,6 +110,10 @@ void Norm::linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int e
     lin(h, out, epilogue, kv, s);
 }
 
+void Norm::add_scaled(const Tensor2&, const float*, float, const Tensor2&, bool, hipStream_t) const {
+    fail("this kind of norm cannot stand behind a sub-layer (it has no scaled add)");
+}
+
 const Tensor2& NormedInput::tensor(Arena& arena, hipStream_t s) {
     if (!have_) {
         h_ = norm_->forward(x_, nullptr, static_cast<int>(x_.rows), arena, s);
@@ -435,9 +439,12 @@ void register_builtin_parts() {
     norms().kinds["layernorm"] = [](const Params& p) { return std::unique_ptr<Norm>(new LayerNorm(p)); };
     mixers().kinds["causal_attention"] = [](const Params& p) { return std::unique_ptr<Mixer>(new CausalSelfAttention(p)); };
     feed_forwards().kinds["dense_mlp"] = [](const Params& p) { return std::unique_ptr<FeedForward>(new DenseMLP(p)); };
-    blocks().kinds["pre_norm"] = [](std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> n) {
+    blocks().kinds["pre_norm"] = [](std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> n, const Params&) {
         return std::unique_ptr<Block>(new PreNormBlock(std::move(m), std::move(f), std::move(n)));
     };
+    register_gated_parts();
+    register_mamba2();
+    register_latent_attention();
 }
 }  // namespace
 
@@ -486,9 +493,9 @@ std::unique_ptr<FeedForward> build_feed_forward(const std::string& kind, const P
     return feed_forwards().get(kind)(p);
 }
 std::unique_ptr<Block> build_block(const std::string& kind, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
-                                   std::vector<std::unique_ptr<Norm>> n) {
+                                   std::vector<std::unique_ptr<Norm>> n, const Params& params) {
     register_builtin_parts();
-    return blocks().get(kind)(std::move(m), std::move(f), std::move(n));
+    return blocks().get(kind)(std::move(m), std::move(f), std::move(n), params);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -519,8 +526,10 @@ std::vector<CacheNeed> DecoderModel::cache_needs() const {
         // a call that only reads must see the cache as the kind of pages or state it would write itself
         const CacheNeed mine = layers[c.layer]->cache_need(), theirs = needs[c.cache];
         if (mine.kind != theirs.kind || mine.n_kv_heads != theirs.n_kv_heads || mine.head_dim != theirs.head_dim ||
-            mine.state_bytes != theirs.state_bytes)
+            mine.value_dim != theirs.value_dim || mine.state_bytes != theirs.state_bytes)
             fail("layer %d reads cache %d, which another kind of mixer writes", c.layer, c.cache);
+        // the pages are kept for the widest window among the calls that read them (0: every key)
+        if (theirs.kind == 1 && theirs.window > 0) needs[c.cache].window = mine.window > 0 ? std::max(theirs.window, mine.window) : 0;
     }
     return needs;
 }

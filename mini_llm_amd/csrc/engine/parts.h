@@ -113,6 +113,7 @@ struct CacheView {
 struct CacheNeed {
     int kind = 0;                        // 1 keys and values in pages, 2 fixed-size state, 0 none
     int n_kv_heads = 0, head_dim = 0, window = 0;
+    int value_dim = -1;                  // width of a head's value rows; -1: as the keys; 0: the pages hold key rows only
     size_t state_bytes = 0;
 };
 
@@ -198,6 +199,10 @@ public:
     // (kv: a key/value scatter of the linear map, passed through to it)
     virtual void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,
                         const KvScatter* kv, Arena& arena, hipStream_t s) const;
+    // x += mult * scale * norm(y), row by row (y and x fp32 [rows, size]; scale per column or null); with
+    // `clear`, y is zero afterwards. For arrangements with a norm behind a sub-layer; a norm without it refuses.
+    virtual void add_scaled(const Tensor2& y, const float* scale, float mult, const Tensor2& x, bool clear,
+                            hipStream_t s) const;
     virtual size_t workspace_bytes(int rows) const = 0;
     virtual void add_cost(StepCost&) const {}
     int dtype = BF16;
@@ -271,8 +276,9 @@ using HeadFactory = std::function<std::unique_ptr<Head>(const Params&)>;
 using NormFactory = std::function<std::unique_ptr<Norm>(const Params&)>;
 using MixerFactory = std::function<std::unique_ptr<Mixer>(const Params&)>;
 using FeedForwardFactory = std::function<std::unique_ptr<FeedForward>(const Params&)>;
+// (the parameters are the arrangement's own: scales, multipliers; "pre_norm" has none)
 using BlockFactory = std::function<std::unique_ptr<Block>(std::unique_ptr<Mixer>, std::unique_ptr<FeedForward>,
-                                                         std::vector<std::unique_ptr<Norm>>)>;
+                                                         std::vector<std::unique_ptr<Norm>>, const Params&)>;
 void register_position(const std::string& kind, PositionFactory f);
 void register_embedding(const std::string& kind, EmbeddingFactory f);
 void register_head(const std::string& kind, HeadFactory f);
@@ -290,7 +296,13 @@ std::unique_ptr<Mixer> build_mixer(const std::string& kind, const Params& p);
 std::unique_ptr<FeedForward> build_feed_forward(const std::string& kind, const Params& p);
 // (the feed-forward may be null: a layer without one; the norms are those of the sub-layers that exist)
 std::unique_ptr<Block> build_block(const std::string& kind, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
-                                   std::vector<std::unique_ptr<Norm>> norms);
+                                   std::vector<std::unique_ptr<Norm>> norms, const Params& params = Params());
+// Parts in files of their own, registered with the built-in ones: RMS norm, the arrangement with a norm on
+// both sides of a sub-layer, the clamped gated feed-forward (parts_gated.cc); the Mamba-2 mixer (mamba2.cc);
+// latent attention (latent_attention.cc).
+void register_gated_parts();
+void register_mamba2();
+void register_latent_attention();
 
 // One entry of the execution order: which layer runs, on which cache, and whether it writes it.
 struct LayerCall {

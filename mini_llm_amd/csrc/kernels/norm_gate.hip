@@ -1,0 +1,171 @@
+// RMS norms (plain, grouped, gated), the normed and scaled residual add, the clamped gated activation
+// and a fill, for gfx950. Statistics and sums are fp32 whatever the activation dtype.
+#include <algorithm>
+
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float sigmoid_precise(float v) { return 1.f / (1.f + expf(-v)); }
+
+// One wavefront per (row, group): y[r, g*Dg + i] = v_i / sqrt(mean_i(v_i^2) + eps) * w[g*Dg + i], with
+// v = x[src row, g*Dg + i] (times silu(gate[row, g*Dg + i]) when a gate is given: the gate comes before
+// the norm). `rows` (optional) selects the input rows. WAVES (row, group) pairs per workgroup.
+template <typename OutT, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
+rmsnorm_kernel(const float* __restrict__ x, int ldx, const int* __restrict__ rows, const float* __restrict__ w,
+               const float* __restrict__ gate, int ldg, OutT* __restrict__ y, int ldy, int n, int D, int groups,
+               float eps) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
+    const long long pair = static_cast<long long>(blockIdx.x) * WAVES + wave;
+    if (pair >= static_cast<long long>(n) * groups) return;
+    const int r = static_cast<int>(pair / groups), g = static_cast<int>(pair % groups), Dg = D / groups;
+    const int src = rows ? rows[r] : r;
+    const float* xr = x + static_cast<size_t>(src) * ldx + g * Dg;
+    const float* gr = gate ? gate + static_cast<size_t>(src) * ldg + g * Dg : nullptr;
+    const float* wr = w + g * Dg;
+    OutT* yr = y + static_cast<size_t>(r) * ldy + g * Dg;
+    // up to 8 elements a lane stay in registers; longer rows are read again
+    float v[8];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int i = lane + 64 * u;
+        float a = 0.f;
+        if (i < Dg) {
+            a = xr[i];
+            if (gr) { const float z = gr[i]; a *= z * sigmoid_precise(z); }
+        }
+        v[u] = a;
+        ss += a * a;
+    }
+    for (int i = lane + 512; i < Dg; i += 64) {
+        float a = xr[i];
+        if (gr) { const float z = gr[i]; a *= z * sigmoid_precise(z); }
+        ss += a * a;
+    }
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(Dg) + eps);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int i = lane + 64 * u;
+        if (i < Dg) yr[i] = from_float<OutT>(v[u] * inv * wr[i]);
+    }
+    for (int i = lane + 512; i < Dg; i += 64) {
+        float a = xr[i];
+        if (gr) { const float z = gr[i]; a *= z * sigmoid_precise(z); }
+        yr[i] = from_float<OutT>(a * inv * wr[i]);
+    }
+}
+
+// x[r, i] += mult * scale[i] * (y[r, i] / sqrt(mean(y[r]^2) + eps) * w[i]); one wavefront per row.
+// With `clear` the row of y is set to zero behind the read, ready to collect the next sub-layer's output.
+template <int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
+rmsnorm_add_kernel(float* __restrict__ y, const float* __restrict__ w, const float* __restrict__ scale, float mult,
+                   float eps, float* __restrict__ x, int n, int D, int clear) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
+    const int r = blockIdx.x * WAVES + wave;
+    if (r >= n) return;
+    float* yr = y + static_cast<size_t>(r) * D;
+    float* xr = x + static_cast<size_t>(r) * D;
+    float v[8];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int i = lane + 64 * u;
+        v[u] = i < D ? yr[i] : 0.f;
+        ss += v[u] * v[u];
+    }
+    for (int i = lane + 512; i < D; i += 64) ss += yr[i] * yr[i];
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(D) + eps);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int i = lane + 64 * u;
+        if (i < D) {
+            const float s = scale ? scale[i] * mult : mult;
+            xr[i] += s * (v[u] * inv * w[i]);
+            if (clear) yr[i] = 0.f;
+        }
+    }
+    for (int i = lane + 512; i < D; i += 64) {
+        const float s = scale ? scale[i] * mult : mult;
+        xr[i] += s * (yr[i] * inv * w[i]);
+        if (clear) yr[i] = 0.f;
+    }
+}
+
+// out[t, i] = g sigmoid(alpha g) (u + 1) with g = min(gate[t, i], limit), u = clamp(up[t, i], -limit, limit).
+template <typename T>
+__global__ void glu_clamped_kernel(const T* gate, int ldg, const T* up, int ldu, T* out, int ldo,     // (out may be gate)
+                                   long long total, int F, float limit, float alpha) {
+    const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int t = static_cast<int>(i / F), f = static_cast<int>(i % F);
+    const float g = fminf(to_float(gate[static_cast<size_t>(t) * ldg + f]), limit);
+    const float u = fminf(fmaxf(to_float(up[static_cast<size_t>(t) * ldu + f]), -limit), limit);
+    const float s = sizeof(T) == 4 ? sigmoid_precise(alpha * g) : __builtin_amdgcn_rcpf(1.f + __expf(-alpha * g));
+    out[static_cast<size_t>(t) * ldo + f] = from_float<T>(g * s * (u + 1.f));
+}
+
+__global__ void fill_zero_kernel(float4* __restrict__ p, size_t n4) {
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n4;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x)
+        p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+}  // namespace
+
+extern "C" {
+
+// y = rmsnorm(x[rows]) in `groups` equal parts of the D columns, optionally gated (see the kernel).
+// x and gate fp32 with row strides ldx / ldg; y in out_dtype with row stride ldy. -1: D is no multiple of groups.
+int mllm_rmsnorm(const float* x, int ldx, const int* rows, const float* w, const float* gate, int ldg, void* y, int ldy,
+                 int n, int D, int groups, float eps, int out_dtype, hipStream_t stream) {
+    if (n <= 0 || D <= 0) return 0;
+    if (groups < 1 || D % groups != 0) return -1;
+    const long long pairs = static_cast<long long>(n) * groups;
+    const int blocks = static_cast<int>((pairs + 3) / 4);
+    if (out_dtype == MLLM_F32)
+        rmsnorm_kernel<float, 4><<<blocks, 256, 0, stream>>>(x, ldx, rows, w, gate, ldg, static_cast<float*>(y), ldy, n, D, groups, eps);
+    else
+        rmsnorm_kernel<bf16_t, 4><<<blocks, 256, 0, stream>>>(x, ldx, rows, w, gate, ldg, static_cast<bf16_t*>(y), ldy, n, D, groups, eps);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+int mllm_rmsnorm_add(float* y, const float* w, const float* scale, float mult, float eps, float* x, int n, int D,
+                     int clear, hipStream_t stream) {
+    if (n <= 0 || D <= 0) return 0;
+    rmsnorm_add_kernel<4><<<(n + 3) / 4, 256, 0, stream>>>(y, w, scale, mult, eps, x, n, D, clear);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+int mllm_glu_clamped(const void* gate, int ldg, const void* up, int ldu, void* out, int ldo, int T, int F, float limit,
+                     float alpha, int dtype, hipStream_t stream) {
+    if (T <= 0 || F <= 0) return 0;
+    const long long total = static_cast<long long>(T) * F;
+    const int blocks = static_cast<int>((total + 255) / 256);
+    if (dtype == MLLM_F32)
+        glu_clamped_kernel<float><<<blocks, 256, 0, stream>>>(static_cast<const float*>(gate), ldg, static_cast<const float*>(up), ldu,
+                                                              static_cast<float*>(out), ldo, total, F, limit, alpha);
+    else
+        glu_clamped_kernel<bf16_t><<<blocks, 256, 0, stream>>>(static_cast<const bf16_t*>(gate), ldg, static_cast<const bf16_t*>(up), ldu,
+                                                               static_cast<bf16_t*>(out), ldo, total, F, limit, alpha);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+// Clears `bytes` bytes (a multiple of 16, the address 16-byte aligned; -1 otherwise) with a kernel, so that
+// the call may be captured into a graph.
+int mllm_fill_zero(void* p, size_t bytes, hipStream_t stream) {
+    if (bytes == 0) return 0;
+    if (bytes % 16 != 0 || (reinterpret_cast<uintptr_t>(p) & 15)) return -1;
+    const size_t n4 = bytes / 16;
+    const int blocks = static_cast<int>(std::min<size_t>((n4 + 255) / 256, 2048));
+    fill_zero_kernel<<<blocks, 256, 0, stream>>>(static_cast<float4*>(p), n4);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"
