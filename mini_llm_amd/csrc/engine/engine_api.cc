@@ -59,7 +59,8 @@ unsigned long long mllm_scratch_bytes(void) {
     return n;
 }
 int mllm_release_scratch(hipStream_t stream) { return guarded([&] { release_scratch(stream); }); }
-// name: "decode_shape" (nsplit, waves; 0, 0 = automatic), "unmerged_shape", "merge_max_rows" (a), "ln_fuse_max_rows" (a), "long_context_splits" (a: 0 off, 1 on)
+// name: "decode_shape" (nsplit, waves; 0, 0 = automatic), "unmerged_shape", "merge_max_rows" (a), "ln_fuse_max_rows" (a), "long_context_splits" (a: 0 off, 1 on),
+// "latent_tiles" (a: 0 off, 1 on)
 int mllm_set_tuning(const char* name, int a, int b) {
     return guarded([&] {
         Tuning& t = tuning();
@@ -69,13 +70,15 @@ int mllm_set_tuning(const char* name, int a, int b) {
         else if (n == "merge_max_rows") t.merge_max_rows = a;
         else if (n == "ln_fuse_max_rows") t.ln_fuse_max_rows = a;
         else if (n == "long_context_splits") t.long_context_splits = a;
+        else if (n == "latent_tiles") t.latent_tiles = a;
         else if (n == "reset_seen") t.seen = Tuning::Seen();
         else fail("unknown tuning value '%s'", name);
     });
 }
 // What the ops chose since the last "reset_seen": "max_decode_splits" (most workgroups a (token, head) pair's keys
 // were split over), "merge_kernel_launches", "prefill_tile_launches" (the bfloat16 matrix-core kernel), "tiled_f32_launches" (the 32-bit one),
-// "generic_attention_launches". -1: unknown name.
+// "generic_attention_launches", "latent_tile_launches" and "latent_token_launches" (latent attention on the matrix cores / one
+// workgroup per token). -1: unknown name.
 long long mllm_get_seen(const char* name) {
     const Tuning::Seen& s = tuning().seen;
     const std::string n(name);
@@ -84,6 +87,8 @@ long long mllm_get_seen(const char* name) {
     if (n == "prefill_tile_launches") return s.prefill_tile_launches;
     if (n == "tiled_f32_launches") return s.tiled_f32_launches;
     if (n == "generic_attention_launches") return s.generic_attention_launches;
+    if (n == "latent_tile_launches") return s.latent_tile_launches;
+    if (n == "latent_token_launches") return s.latent_token_launches;
     return -1;
 }
 

@@ -78,13 +78,16 @@ int mllm_ssm_scan(const float* xbc, int ldx, const float* raw_dt, int ldd, const
 
 // latent_attention.hip
 int mllm_latent_prepare(const float* dq, int ld_dq, int Rq, const float* wq, void* cq, int ld_cq, const float* dkv, int ld_dkv,
-                        int R, int Dr, const float* wkv, void* pages, const int* slots, const int* positions, int T, float eps,
-                        double base, int rot_dims, int dtype, hipStream_t stream);
+                        int R, int Dr, const float* wkv, void* pages, void* vt_pages, int page_size, const int* slots,
+                        const int* positions, int T, float eps, double base, int rot_dims, int dtype, hipStream_t stream);
 int mllm_latent_absorb(const void* q, int ldq, const void* w_uk, int ldw, void* qa, int ldqa, const int* positions, int T, int H,
                        int Dn, int Dr, int R, double base, int rot_dims, int dtype, hipStream_t stream);
 int mllm_latent_attention(const void* qa, int ldqa, const void* pages, const int* block_tables, int max_blocks,
                           const int* token_seq, const int* positions, int T, int H, int R, int Dr, int page_size, float scale,
                           int window, void* o_lat, int ldo, int dtype, hipStream_t stream);
+int mllm_latent_attention_tiles(const void* qa, const void* k_pages, const void* vt_pages, const int* block_tables,
+                                int max_blocks, const int* cu_q, const int* ctx_len, int n_seqs, int n_tiles_upper, int H,
+                                int R, int Dr, int page_size, float scale, int window, void* o_lat, hipStream_t stream);
 int mllm_latent_expand(const void* o_lat, int ldo, const void* w_uv, int ldw, void* out, int ldout, int T, int H, int Dv, int R,
                        int dtype, hipStream_t stream);
 

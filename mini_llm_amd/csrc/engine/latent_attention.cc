@@ -17,7 +17,8 @@ const float* f32_vector(const Params& p, const char* key, int n) {
 //   W_dkv h = [kv_rank | rot_dim]:  c = rmsnorm(first part) * w_dkvn,  k_rot = the second part, turned
 //   per head: k = W_uk c, v = W_uv c;  score = scale * (q_plain . k + turned(q_rot) . k_rot), causal within
 //   `window` (0: none), softmax;  out = W_o concat_heads(sum_j p_j v_j), added into the stream.
-// The pages hold rows [c | k_rot] and nothing per head. The kernels work in the latent's space
+// The pages hold rows [c | k_rot] and nothing per head (in bfloat16 also c once more, transposed page by page,
+// the operand shape of the matrix-core kernel for prompt portions). The kernels work in the latent's space
 // (kernels/latent_attention.hip): the plain part of a query is multiplied by W_uk^T first, attention runs
 // over the page rows with the first kv_rank columns as values, and W_uv expands the result.
 // A mixer without the tensor "dkv.weight" reads pages that another layer's call has written (its execution
@@ -81,15 +82,19 @@ public:
             dkv = arena.tensor(F32, T, E);
             dkv_(in, dkv, STORE_F32, nullptr, s);
         }
-        latent_prepare(dq, dq_norm_, cq, fill ? &dkv : nullptr, dkv_norm_, fill ? &cache.k_pages : nullptr, step.slots[g], step.positions, sh_, s);
+        LatentPages pages;
+        pages.rows = cache.k_pages; pages.latent_t = cache.v_pages; pages.page_size = cache.page_size;
+        latent_prepare(dq, dq_norm_, cq, fill ? &dkv : nullptr, dkv_norm_, fill ? &pages : nullptr, step.slots[g], step.positions, sh_, s);
         Tensor2 q = arena.tensor(dtype_, T, H * (sh_.plain_dim + sh_.rot_dim));
         uq_(cq, q, STORE, nullptr, s);
         Tensor2 qa = arena.tensor(dtype_, T, H * E);
         latent_absorb(q, uk_, qa, step.positions, sh_, s);
         StageTimes::get().mark("qkv", s);
         Tensor2 o_lat = arena.tensor(dtype_, T, H * sh_.kv_rank);
-        latent_attention(qa, cache.k_pages, cache.page_size, step.block_tables[g], step.max_blocks[g], step.token_seq, step.positions,
-                         scale_, window_, sh_, o_lat, s);
+        LatentStep ls;
+        ls.block_tables = step.block_tables[g]; ls.max_blocks = step.max_blocks[g]; ls.n_seqs = step.n_seqs; ls.max_q_len = step.max_q_len;
+        ls.token_seq = step.token_seq; ls.positions = step.positions; ls.cu_q = step.cu_q; ls.ctx_len = step.ctx_len;
+        latent_attention(qa, pages, ls, scale_, window_, sh_, o_lat, s);
         StageTimes::get().mark("attention", s);
         Tensor2 o = arena.tensor(dtype_, T, H * sh_.value_dim);
         latent_expand(o_lat, uv_, o, sh_, s);
@@ -103,7 +108,9 @@ public:
     }
     CacheNeed cache_need() const override {
         CacheNeed n;
-        n.kind = 1; n.n_kv_heads = 1; n.head_dim = sh_.kv_rank + sh_.rot_dim; n.value_dim = 0; n.window = window_;
+        // (the "value" pool holds the latent once more, transposed page by page, for the matrix-core kernel:
+        // only the bfloat16 path has that kernel)
+        n.kind = 1; n.n_kv_heads = 1; n.head_dim = sh_.kv_rank + sh_.rot_dim; n.value_dim = dtype_ == BF16 ? sh_.kv_rank : 0; n.window = window_;
         return n;
     }
     void reserve(int, hipStream_t s) const override { reserve_linear_scratch(s); }

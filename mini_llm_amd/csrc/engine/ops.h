@@ -106,10 +106,12 @@ struct Tuning {
     int merge_max_rows = 16;                          // tokens whose splits a product merges while loading
     int long_context_splits = 1;                      // 1: few pairs with long contexts are split over up to 256 workgroups
     int ln_fuse_max_rows = 32;                        // rows up to which the norm is fused into the few-row product
+    int latent_tiles = 1;                             // 1: latent attention's prompt portions may run on the matrix cores
     // what the ops chose since the last reset (tests read it back instead of trusting the thresholds)
     struct Seen {
         int max_decode_splits = 0;                    // most workgroups a (token, head) pair's keys were split over
         long long merge_kernel_launches = 0, prefill_tile_launches = 0, tiled_f32_launches = 0, generic_attention_launches = 0;
+        long long latent_tile_launches = 0, latent_token_launches = 0;      // latent attention: matrix-core kernel, one workgroup per token
     } seen;
 };
 Tuning& tuning();
@@ -192,16 +194,33 @@ struct LatentShape {
     double rot_base = 10000.0;
     float eps = 1e-6f;
 };
+// The pages of latent attention: `rows` [n_pages * page_size, kv_rank + rot_dim] holds a row [c | k_rot] per
+// token; `latent_t` (optional, [n_pages * page_size, kv_rank] in size) holds c once more, transposed page by
+// page ([page][kv_rank][page_size]): the operand shape of the matrix-core kernel.
+struct LatentPages {
+    Tensor2 rows, latent_t;
+    int page_size = 0;
+};
 // cq = rmsnorm(dq) * wq; with dkv: page row slots[t] = [rmsnorm(dkv[:, :kv_rank]) * wkv | turned rest]
 void latent_prepare(const Tensor2& dq, const float* wq, const Tensor2& cq, const Tensor2* dkv, const float* wkv,
-                    const Tensor2* pages, const int* slots, const int* positions, const LatentShape& sh, hipStream_t stream);
+                    const LatentPages* pages, const int* slots, const int* positions, const LatentShape& sh, hipStream_t stream);
 // qa[t, h] = [W_uk_h^T q_plain[t, h] | turned q_rot[t, h]]
 void latent_absorb(const Tensor2& q, const Tensor2& w_uk, const Tensor2& qa, const int* positions, const LatentShape& sh,
                    hipStream_t stream);
-// o_lat[t, h] = sum_j softmax_j(scale * qa[t, h] . row_j) row_j[:kv_rank] over the visible rows of the pages
-void latent_attention(const Tensor2& qa, const Tensor2& pages, int page_size, const int* block_tables, int max_blocks,
-                      const int* token_seq, const int* positions, float scale, int window, const LatentShape& sh,
-                      const Tensor2& o_lat, hipStream_t stream);
+// The step's sequences, as attention sees them.
+struct LatentStep {
+    const int* block_tables = nullptr;     // [n_seqs, max_blocks]
+    int max_blocks = 0, n_seqs = 0, max_q_len = 0;
+    const int* token_seq = nullptr;        // [T]
+    const int* positions = nullptr;        // [T]
+    const int* cu_q = nullptr;             // [n_seqs + 1]
+    const int* ctx_len = nullptr;          // [n_seqs]
+};
+// o_lat[t, h] = sum_j softmax_j(scale * qa[t, h] . row_j) row_j[:kv_rank] over the visible rows of the pages.
+// Steps with prompt portions run on the matrix cores where the sizes allow (bfloat16, the transposed latent
+// at hand), others one workgroup per token.
+void latent_attention(const Tensor2& qa, const LatentPages& pages, const LatentStep& step, float scale, int window,
+                      const LatentShape& sh, const Tensor2& o_lat, hipStream_t stream);
 // out[t, h*value_dim + e] = sum_r w_uv[h*value_dim + e, r] * o_lat[t, h, r]
 void latent_expand(const Tensor2& o_lat, const Tensor2& w_uv, const Tensor2& out, const LatentShape& sh, hipStream_t stream);
 

@@ -117,8 +117,18 @@ static void check_shape(const LatentShape& sh, const char* what) {
         fail("%s: %d of %d rotary columns (both even) and a positive base are needed", what, sh.rot_dims, sh.rot_dim);
 }
 
+static void check_pages(const LatentPages& pages, int dtype, const LatentShape& sh, const char* what) {
+    const int E = sh.kv_rank + sh.rot_dim;
+    if (pages.rows.dtype != dtype || !pages.rows.contiguous() || pages.rows.cols != E)
+        fail("%s: the pages must be contiguous [rows, %d] %s", what, E, dtype_name(dtype));
+    if (pages.page_size < 1 || pages.rows.rows % pages.page_size != 0) fail("%s: the page pool is not a whole number of pages", what);
+    if (pages.latent_t.data != nullptr &&
+        (pages.latent_t.dtype != dtype || !pages.latent_t.contiguous() || pages.latent_t.cols != sh.kv_rank || pages.latent_t.rows != pages.rows.rows))
+        fail("%s: the transposed latent must be contiguous [rows, %d] %s", what, sh.kv_rank, dtype_name(dtype));
+}
+
 void latent_prepare(const Tensor2& dq, const float* wq, const Tensor2& cq, const Tensor2* dkv, const float* wkv,
-                    const Tensor2* pages, const int* slots, const int* positions, const LatentShape& sh, hipStream_t stream) {
+                    const LatentPages* pages, const int* slots, const int* positions, const LatentShape& sh, hipStream_t stream) {
     check_shape(sh, "latent_prepare");
     need_f32(dq, "latent_prepare: the query latent");
     need_act(cq, "latent_prepare: cq");
@@ -128,12 +138,12 @@ void latent_prepare(const Tensor2& dq, const float* wq, const Tensor2& cq, const
         need_f32(*dkv, "latent_prepare: the key/value latent");
         if (pages == nullptr || slots == nullptr || positions == nullptr || wkv == nullptr) fail("latent_prepare: pages, page rows, positions and the norm weight are needed");
         if (dkv->cols != sh.kv_rank + sh.rot_dim || dkv->rows != dq.rows) fail("latent_prepare: the key/value latent must be [T, %d]", sh.kv_rank + sh.rot_dim);
-        if (pages->dtype != cq.dtype || !pages->contiguous() || pages->cols != sh.kv_rank + sh.rot_dim)
-            fail("latent_prepare: the pages must be contiguous [rows, %d] %s", sh.kv_rank + sh.rot_dim, dtype_name(cq.dtype));
+        check_pages(*pages, cq.dtype, sh, "latent_prepare");
     }
     check(mllm_latent_prepare(static_cast<const float*>(dq.data), i32(dq.stride), sh.q_rank, wq, cq.data, i32(cq.stride),
                               dkv ? static_cast<const float*>(dkv->data) : nullptr, dkv ? i32(dkv->stride) : 0, sh.kv_rank, sh.rot_dim, wkv,
-                              dkv ? pages->data : nullptr, slots, positions, i32(dq.rows), sh.eps, sh.rot_base, sh.rot_dims, cq.dtype, stream),
+                              dkv ? pages->rows.data : nullptr, dkv ? pages->latent_t.data : nullptr, dkv ? pages->page_size : 0, slots, positions,
+                              i32(dq.rows), sh.eps, sh.rot_base, sh.rot_dims, cq.dtype, stream),
           "latent_prepare");
 }
 
@@ -151,22 +161,34 @@ void latent_absorb(const Tensor2& q, const Tensor2& w_uk, const Tensor2& qa, con
                              sh.plain_dim, sh.rot_dim, sh.kv_rank, sh.rot_base, sh.rot_dims, q.dtype, stream), "latent_absorb");
 }
 
-void latent_attention(const Tensor2& qa, const Tensor2& pages, int page_size, const int* block_tables, int max_blocks,
-                      const int* token_seq, const int* positions, float scale, int window, const LatentShape& sh,
-                      const Tensor2& o_lat, hipStream_t stream) {
+void latent_attention(const Tensor2& qa, const LatentPages& pages, const LatentStep& step, float scale, int window,
+                      const LatentShape& sh, const Tensor2& o_lat, hipStream_t stream) {
     check_shape(sh, "latent_attention");
     need_act(qa, "latent_attention: qa");
-    const int E = sh.kv_rank + sh.rot_dim;
+    const int E = sh.kv_rank + sh.rot_dim, T = i32(qa.rows);
     if (qa.cols != static_cast<int64_t>(sh.n_heads) * E) fail("latent_attention: qa must be [T, %d]", sh.n_heads * E);
-    if (pages.dtype != qa.dtype || !pages.contiguous() || pages.cols != E) fail("latent_attention: the pages must be contiguous [rows, %d] %s", E, dtype_name(qa.dtype));
-    if (page_size < 1 || pages.rows % page_size != 0) fail("latent_attention: the page pool is not a whole number of pages");
+    check_pages(pages, qa.dtype, sh, "latent_attention");
     if (o_lat.dtype != qa.dtype || o_lat.rows != qa.rows || o_lat.cols != static_cast<int64_t>(sh.n_heads) * sh.kv_rank)
         fail("latent_attention: the result must be [T, %d]", sh.n_heads * sh.kv_rank);
-    if (block_tables == nullptr || token_seq == nullptr || positions == nullptr || max_blocks < 1) fail("latent_attention: block tables, token_seq and positions are needed");
+    if (step.block_tables == nullptr || step.token_seq == nullptr || step.positions == nullptr || step.max_blocks < 1)
+        fail("latent_attention: block tables, token_seq and positions are needed");
     if (qa.dtype == BF16 && E % 2 != 0) fail("latent_attention: rows of %d bfloat16 columns are not supported (an even number is)", E);
     if (window < 0) fail("latent_attention: a negative window");
-    check(mllm_latent_attention(qa.data, i32(qa.stride), pages.data, block_tables, max_blocks, token_seq, positions, i32(qa.rows), sh.n_heads,
-                                sh.kv_rank, sh.rot_dim, page_size, scale, window, o_lat.data, i32(o_lat.stride), qa.dtype, stream),
+    // prompt portions: the matrix-core kernel, one workgroup per 64 (token, head) rows of a sequence
+    if (tuning().latent_tiles && step.max_q_len > 1 && qa.dtype == BF16 && pages.latent_t.data != nullptr && step.cu_q != nullptr &&
+        step.ctx_len != nullptr && step.n_seqs > 0 && qa.contiguous() && o_lat.contiguous()) {
+        const long long tiles = static_cast<long long>(T) * sh.n_heads / 64 + step.n_seqs;
+        if (tiles < (1ll << 31)) {
+            const int rc = mllm_latent_attention_tiles(qa.data, pages.rows.data, pages.latent_t.data, step.block_tables, step.max_blocks, step.cu_q,
+                                                       step.ctx_len, step.n_seqs, static_cast<int>(tiles), sh.n_heads, sh.kv_rank, sh.rot_dim,
+                                                       pages.page_size, scale, window, o_lat.data, stream);
+            if (rc == 0) { tuning().seen.latent_tile_launches += 1; return; }
+            if (rc != -2) check(rc, "latent_attention (tiles)");
+        }
+    }
+    tuning().seen.latent_token_launches += 1;
+    check(mllm_latent_attention(qa.data, i32(qa.stride), pages.rows.data, step.block_tables, step.max_blocks, step.token_seq, step.positions, T,
+                                sh.n_heads, sh.kv_rank, sh.rot_dim, pages.page_size, scale, window, o_lat.data, i32(o_lat.stride), qa.dtype, stream),
           "latent_attention");
 }
 

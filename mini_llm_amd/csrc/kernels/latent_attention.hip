@@ -23,14 +23,14 @@ __device__ __forceinline__ void turn_pair(float u, float v, int pos, int i, doub
 
 // One wavefront per token:
 //   cq[t]  = rmsnorm(dq[t]) * wq                                      (the query latent, activation dtype)
-//   page row slots[t] = [ rmsnorm(dkv[t, :R]) * wkv | turned dkv[t, R:R+Dr] ]   (if dkv is given and slot >= 0)
+//   page row slots[t] = [ c = rmsnorm(dkv[t, :R]) * wkv | turned dkv[t, R:R+Dr] ]   (if dkv is given and slot >= 0)
 // The first rot_dims of the Dr columns are turned in interleaved pairs, the rest pass unchanged.
 template <typename T>
 __global__ void __launch_bounds__(64)
 latent_prepare_kernel(const float* __restrict__ dq, int ld_dq, int Rq, const float* __restrict__ wq, T* __restrict__ cq,
                       int ld_cq, const float* __restrict__ dkv, int ld_dkv, int R, int Dr, const float* __restrict__ wkv,
-                      T* __restrict__ pages, const int* __restrict__ slots, const int* __restrict__ positions, float eps,
-                      double log2_base, int rot_dims) {
+                      T* __restrict__ pages, T* __restrict__ vt_pages, int page_size, const int* __restrict__ slots,
+                      const int* __restrict__ positions, float eps, double log2_base, int rot_dims) {
     const int t = blockIdx.x, lane = threadIdx.x;
     {
         const float* row = dq + static_cast<size_t>(t) * ld_dq;
@@ -48,7 +48,14 @@ latent_prepare_kernel(const float* __restrict__ dq, int ld_dq, int Rq, const flo
     float ss = 0.f;
     for (int i = lane; i < R; i += 64) ss += row[i] * row[i];
     const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(R) + eps);
-    for (int i = lane; i < R; i += 64) o[i] = from_float<T>(row[i] * inv * wkv[i]);
+    // (vt_pages, optional: the latent once more, transposed page by page, [page][R][page_size], which is the
+    // operand shape of the matrix-core kernel's second product)
+    T* vt = vt_pages ? vt_pages + static_cast<size_t>(slot / page_size) * page_size * R + slot % page_size : nullptr;
+    for (int i = lane; i < R; i += 64) {
+        const T c = from_float<T>(row[i] * inv * wkv[i]);
+        o[i] = c;
+        if (vt) vt[static_cast<size_t>(i) * page_size] = c;
+    }
     const int pos = positions[t];
     for (int i = lane; i < rot_dims / 2; i += 64) {
         float a, b;
@@ -221,6 +228,172 @@ latent_expand_kernel(const T* __restrict__ o_lat, int ldo, const T* __restrict__
     }
 }
 
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+union Frag8 {
+    bf16x8 v;
+    u32x4 q;
+    uint32_t w[4];
+};
+
+// Prompt portions on the matrix cores (bfloat16, fp32 softmax). A query row is a (token, head) pair; a
+// sequence's rows are numbered token by token, head by head, and a workgroup takes 64 consecutive rows (its
+// four wavefronts 16 each), which lie on few neighbouring tokens, so they share their keys: one staging of a
+// 64-key tile serves all of them. Everything is computed transposed, one query row per lane, as in the
+// framework's other prompt-attention kernel (attention_prefill.hip):
+//   S^T = K Q^T    A = 16 page rows x 32 columns from LDS, B = the lane's absorbed query, in registers
+//   O^T = C^T P^T  A = 16 latent columns x 32 keys, B = P^T straight from the S^T accumulators
+// The second product's A operand needs 8 keys of one latent column side by side, which the page-transposed
+// copy of the latent holds ([page][R][page_size]): its 16-byte pieces go to LDS as they are, keys outside
+// the tile's range set to zero (a page's tail may hold anything). E = 32 * KS, R = 16 * DT.
+template <int KS, int DT>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2)))
+latent_prefill_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
+                      const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
+                      const int* __restrict__ ctx_len, int n_seqs, int H, int page_size, float scale_log2e, int window,
+                      bf16_t* __restrict__ o_lat) {
+    constexpr int E = 32 * KS, R = 16 * DT, BN = 64, KSTRIDE = E + 8, VSTRIDE = BN + 8, CH = E / 8;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    bf16_t* Ks = reinterpret_cast<bf16_t*>(smem);                    // [BN][KSTRIDE]
+    bf16_t* Vt = Ks + BN * KSTRIDE;                                  // [R][VSTRIDE]
+    int* sm_table = reinterpret_cast<int*>(Vt + R * VSTRIDE);        // the sequence's block table
+
+    int tile = gridDim.x - 1 - blockIdx.x, b = 0, q_begin = 0, q_len = 0;
+    for (; b < n_seqs; ++b) {
+        q_begin = cu_q[b];
+        q_len = cu_q[b + 1] - q_begin;
+        const int nt = (q_len * H + 63) / 64;
+        if (tile < nt) break;
+        tile -= nt;
+    }
+    if (b >= n_seqs) return;                       // surplus workgroup; the whole workgroup leaves
+    const int tid = threadIdx.x, lane = tid % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int G = lane / 16, c16 = lane % 16;
+    const int rows = q_len * H, start = ctx_len[b] - q_len;
+    const int rho0 = tile * 64, rho = rho0 + wave * 16 + c16;
+    const bool q_ok = rho < rows;
+    const int rho_c = min(rho, rows - 1);
+    const int p = start + rho_c / H;                              // this lane's position
+    const int p_first = start + rho0 / H, p_last = start + min(rho0 + 63, rows - 1) / H;
+    const int k_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+    const int shift = __ffs(page_size) - 1;
+    const int* gtable = block_tables + static_cast<size_t>(b) * max_blocks;
+    for (int i = tid; i <= (p_last >> shift); i += 256) sm_table[i] = gtable[i];
+    __syncthreads();
+
+    Frag8 qf[KS];
+    const bf16_t* qrow = qa + (static_cast<size_t>(q_begin) * H + rho_c) * E;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks].q = *reinterpret_cast<const u32x4*>(qrow + 32 * ks + 8 * G);
+
+    float m = -INFINITY, l = 0.f;
+    f32x4 o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int pg_lo = k_lo >> shift, pg_hi = p_last >> shift;
+
+    for (int kt = k_lo / BN; kt <= p_last / BN; ++kt) {
+        const int j_base = kt * BN;
+        __syncthreads();                           // the tile before is used up
+        // page rows, row-major; a key outside [k_lo, p_last] is replaced by one inside (always a held page;
+        // its scores are masked below)
+        for (int idx = tid; idx < BN * CH; idx += 256) {
+            const int j = idx / CH, c = idx % CH;
+            const int key = min(max(j_base + j, k_lo), p_last);
+            const size_t row = (static_cast<size_t>(sm_table[key >> shift]) << shift) + (key & (page_size - 1));
+            *reinterpret_cast<u32x4*>(Ks + j * KSTRIDE + 8 * c) = *reinterpret_cast<const u32x4*>(k_pages + row * E + 8 * c);
+        }
+        // the latent transposed: 8 keys of one column a piece
+        for (int idx = tid; idx < R * (BN / 8); idx += 256) {
+            const int col = idx / (BN / 8), part = idx % (BN / 8);
+            const int key0 = j_base + 8 * part;
+            const int pg = min(max(key0 >> shift, pg_lo), pg_hi);
+            const bf16_t* src = vt_pages + (static_cast<size_t>(sm_table[pg]) << shift) * R + static_cast<size_t>(col) * page_size +
+                                (key0 & (page_size - 1));
+            u32x4 v = *reinterpret_cast<const u32x4*>(src);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int ka = key0 + 2 * e, kb = ka + 1;
+                const uint32_t keep = ((ka >= k_lo && ka <= p_last) ? 0x0000ffffu : 0u) | ((kb >= k_lo && kb <= p_last) ? 0xffff0000u : 0u);
+                v[e] &= keep;
+            }
+            *reinterpret_cast<u32x4*>(Vt + col * VSTRIDE + 8 * part) = v;
+        }
+        __syncthreads();
+        // S^T: s[nt][r] is the score of key j_base + 16 nt + 4 G + r with this lane's query row
+        float s[4][4];
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const bf16x8 a = *reinterpret_cast<const bf16x8*>(Ks + (16 * nt + c16) * KSTRIDE + 32 * ks + 8 * G);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[ks].v, acc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int j = j_base + 16 * nt + 4 * G + r;
+                const bool seen = q_ok && j <= p && (window <= 0 || j > p - window);
+                s[nt][r] = seen ? acc[r] : -INFINITY;
+                tile_max = fmaxf(tile_max, s[nt][r]);
+            }
+        }
+        tile_max = rows_max(tile_max);             // the four lane groups of a query row agree on the maximum
+        const float m_new = fmaxf(m, tile_max * scale_log2e);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = fast_exp2(m - m_use);
+        m = m_new;
+        float psum = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                s[nt][r] = fast_exp2(fmaf(s[nt][r], scale_log2e, -m_use));
+                psum += s[nt][r];
+            }
+        l = l * alpha + psum;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+        // O^T += C^T P^T over slabs of 32 keys: k slot i of lane group G stands for key 32 slab + 4 G + i
+        // (i < 4) or 32 slab + 16 + 4 G + i - 4 (i >= 4) in both operands
+#pragma unroll
+        for (int slab = 0; slab < 2; ++slab) {
+            Frag8 pf;
+            pf.w[0] = pack_bf16x2(s[2 * slab][0], s[2 * slab][1]);
+            pf.w[1] = pack_bf16x2(s[2 * slab][2], s[2 * slab][3]);
+            pf.w[2] = pack_bf16x2(s[2 * slab + 1][0], s[2 * slab + 1][1]);
+            pf.w[3] = pack_bf16x2(s[2 * slab + 1][2], s[2 * slab + 1][3]);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const uint32_t* vrow = reinterpret_cast<const uint32_t*>(Vt + (16 * dt + c16) * VSTRIDE);
+                Frag8 vf;
+                vf.w[0] = vrow[16 * slab + 2 * G];
+                vf.w[1] = vrow[16 * slab + 2 * G + 1];
+                vf.w[2] = vrow[16 * slab + 8 + 2 * G];
+                vf.w[3] = vrow[16 * slab + 8 + 2 * G + 1];
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
+            }
+        }
+    }
+    l = rows_sum(l);
+    if (!q_ok) return;
+    const float inv = 1.0f / l;
+    // o[dt][r] is latent column 16 dt + 4 G + r of this lane's query row
+    bf16_t* orow = o_lat + (static_cast<size_t>(q_begin) * H + rho) * R;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        uint2 pk;
+        pk.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
+        pk.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
+        *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * G) = pk;
+    }
+}
+
 constexpr int MAX_LDS = 160 * 1024;
 
 }  // namespace
@@ -230,17 +403,19 @@ extern "C" {
 // See latent_prepare_kernel. dkv may be null (a layer that reads another layer's pages). -1: an odd rot_dims
 // or one beyond Dr.
 int mllm_latent_prepare(const float* dq, int ld_dq, int Rq, const float* wq, void* cq, int ld_cq, const float* dkv, int ld_dkv,
-                        int R, int Dr, const float* wkv, void* pages, const int* slots, const int* positions, int T, float eps,
-                        double base, int rot_dims, int dtype, hipStream_t stream) {
+                        int R, int Dr, const float* wkv, void* pages, void* vt_pages, int page_size, const int* slots,
+                        const int* positions, int T, float eps, double base, int rot_dims, int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
-    if (rot_dims < 0 || rot_dims % 2 != 0 || rot_dims > Dr || !(base > 0)) return -1;
+    if (rot_dims < 0 || rot_dims % 2 != 0 || rot_dims > Dr || !(base > 0) || (vt_pages != nullptr && page_size < 1)) return -1;
     const double l2 = log2(base);
     if (dtype == MLLM_F32)
         latent_prepare_kernel<float><<<T, 64, 0, stream>>>(dq, ld_dq, Rq, wq, static_cast<float*>(cq), ld_cq, dkv, ld_dkv, R, Dr, wkv,
-                                                           static_cast<float*>(pages), slots, positions, eps, l2, rot_dims);
+                                                           static_cast<float*>(pages), static_cast<float*>(vt_pages), page_size, slots, positions,
+                                                           eps, l2, rot_dims);
     else
         latent_prepare_kernel<bf16_t><<<T, 64, 0, stream>>>(dq, ld_dq, Rq, wq, static_cast<bf16_t*>(cq), ld_cq, dkv, ld_dkv, R, Dr, wkv,
-                                                            static_cast<bf16_t*>(pages), slots, positions, eps, l2, rot_dims);
+                                                            static_cast<bf16_t*>(pages), static_cast<bf16_t*>(vt_pages), page_size, slots, positions,
+                                                            eps, l2, rot_dims);
     MLLM_LAUNCH_CHECK();
     return 0;
 }
@@ -302,6 +477,43 @@ int mllm_latent_attention(const void* qa, int ldqa, const void* pages, const int
 #undef LATENT_ATTN
     MLLM_LAUNCH_CHECK();
     return 0;
+}
+
+// Prompt portions on the matrix cores (see latent_prefill_kernel): qa [T*H, E] and o_lat [T*H, R] contiguous
+// bfloat16. n_tiles_upper: an upper bound of sum over sequences of ceil(q_len * H / 64). Returns -2 when the
+// sizes are not ones it is built for (E and R among (128, 96), (96, 64), (160, 128), (288, 256), (576, 512);
+// page sizes 8 to 64, powers of two; a block table that fits the LDS beside the tiles): the caller then runs
+// mllm_latent_attention.
+int mllm_latent_attention_tiles(const void* qa, const void* k_pages, const void* vt_pages, const int* block_tables,
+                                int max_blocks, const int* cu_q, const int* ctx_len, int n_seqs, int n_tiles_upper, int H,
+                                int R, int Dr, int page_size, float scale, int window, void* o_lat, hipStream_t stream) {
+    if (n_seqs <= 0 || n_tiles_upper <= 0) return 0;
+    const int E = R + Dr;
+    if (E % 32 != 0 || R % 16 != 0 || page_size < 8 || page_size > 64 || (page_size & (page_size - 1)) != 0) return -2;
+    if (((reinterpret_cast<uintptr_t>(qa) | reinterpret_cast<uintptr_t>(k_pages) | reinterpret_cast<uintptr_t>(vt_pages) |
+          reinterpret_cast<uintptr_t>(o_lat)) & 15) != 0)
+        return -2;
+    const size_t lds = static_cast<size_t>(64) * (E + 8) * 2 + static_cast<size_t>(R) * 72 * 2 + static_cast<size_t>(max_blocks) * 4;
+    if (lds > static_cast<size_t>(MAX_LDS)) return -2;
+    const float sl2 = scale * 1.44269504088896340736f;
+#define LP_CASE(KS, DT)                                                                                              \
+    if (E == 32 * KS && R == 16 * DT) {                                                                              \
+        static bool allowed = false;                                                                                 \
+        if (!allowed) {                                                                                              \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(latent_prefill_kernel<KS, DT>),         \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS);                 \
+            if (e != hipSuccess) return static_cast<int>(e);                                                         \
+            allowed = true;                                                                                          \
+        }                                                                                                            \
+        latent_prefill_kernel<KS, DT><<<n_tiles_upper, 256, lds, stream>>>(                                          \
+            static_cast<const bf16_t*>(qa), static_cast<const bf16_t*>(k_pages), static_cast<const bf16_t*>(vt_pages), \
+            block_tables, max_blocks, cu_q, ctx_len, n_seqs, H, page_size, sl2, window, static_cast<bf16_t*>(o_lat)); \
+        MLLM_LAUNCH_CHECK();                                                                                         \
+        return 0;                                                                                                    \
+    }
+    LP_CASE(4, 6) LP_CASE(3, 4) LP_CASE(5, 8) LP_CASE(9, 16) LP_CASE(18, 32)
+#undef LP_CASE
+    return -2;
 }
 
 int mllm_latent_expand(const void* o_lat, int ldo, const void* w_uv, int ldw, void* out, int ldout, int T, int H, int Dv, int R,

@@ -157,7 +157,7 @@ def scratch_bytes() -> int:
 
 def seen(name: str) -> int:
     """What the ops chose since ``reset_seen()``: "max_decode_splits", "merge_kernel_launches",
-    "prefill_tile_launches", "generic_attention_launches"."""
+    "prefill_tile_launches", "generic_attention_launches", "latent_tile_launches", "latent_token_launches"."""
     v = engine_library().mllm_get_seen(name.encode())
     if v < 0:
         raise KernelError(f"unknown counter '{name}'")
@@ -166,6 +166,11 @@ def seen(name: str) -> int:
 
 def reset_seen() -> None:
     _ok(engine_library().mllm_set_tuning(b"reset_seen", 0, 0))
+
+
+def set_latent_tiles(on: bool) -> None:
+    """Whether latent attention's prompt portions may run on the matrix cores (default: on)."""
+    _ok(engine_library().mllm_set_tuning(b"latent_tiles", 1 if on else 0, 0))
 
 
 # Tuning hooks: tests and tuning scripts set these module attributes; they reach the native side at the

@@ -56,6 +56,16 @@ MIXED_B = model([
 # scores that one key dominates: a window that is one key off, or a key lost at a page's border, changes a row
 PEAKED = model([latent(window=5, scale=6.0), latent(window=16, scale=6.0, heads=1), latent(window=6, scale=6.0, kv_from=1)], width=32)
 
+# cached rows of 96 and 160 columns (latents of 64 and 128): sizes that the matrix-core kernel of prompt portions
+# takes at pages of 16 tokens in bfloat16; windows shorter and longer than its 64-key tiles; 3 and 5 heads, so
+# that a tile of 64 (token, head) rows starts and ends in the middle of a token
+TILED = model([
+    latent(heads=3, dim=16, rot_dim=32, vdim=16, kv_rank=64, q_rank=32, window=40, mlp=dense(64, 1.2)),
+    mamba(heads=4, vdim=8, state=8, groups=2, conv=3, norm_groups=1),
+    latent(heads=5, dim=8, rot_dim=32, vdim=24, kv_rank=128, q_rank=40, window=150),
+    latent(heads=2, dim=24, rot_dim=32, vdim=8, kv_rank=128, q_rank=16, window=70, kv_from=2),
+], vocab=211, width=56, mult=0.6)
+
 # rms(difference, mean taken off) / rms(logits, mean taken off) of a row may be at most this
 TOL = {"float32": 5e-6, "bfloat16": 6e-2}
 # with the peaked scores of PEAKED, 32-bit rounding shows more (seen: 2e-5)

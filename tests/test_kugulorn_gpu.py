@@ -69,6 +69,43 @@ def test_schedule_families_match_plain(dirs, name, family, dtype):
     assert runner.check() == "" and info["free_pages"] == n_pages and info["n_requests"] == 0
 
 
+@pytest.mark.parametrize("page", [8, 16, 64])
+@pytest.mark.parametrize("family", ["whole", "decode", "chunks", "mixed"])
+def test_prompt_portions_on_the_matrix_cores(dirs, family, page):
+    """bfloat16 at sizes and page sizes that the matrix-core kernel takes: prompts of up to 300 tokens (several
+    key tiles, windows that end inside a tile), portions, and mixed batches whose single tokens ride along."""
+    from mini_llm_amd.kernels import ops
+    cfg, d = kc.TILED, dirs("TILED")
+    reqs = kc.requests(cfg["vocab"], [1, 2, 17, 63, 64, 65, 130, 300], seed=71)
+    steps = _families(reqs, seed=6)[family]
+    ops.reset_seen()
+    runner = _runner(d, "bfloat16", n_pages=-(-ru.peak_tokens(steps) // page), page=page)
+    kc.check_against_plain(d, reqs, steps, ru.run_in_process(runner, steps), "bfloat16", cfg["vocab"], f"tiled page {page} {family}")
+    assert ops.seen("latent_tile_launches") > 0
+    assert runner.check() == "" and runner.info()["n_requests"] == 0
+
+
+def test_matrix_core_kernel_against_the_per_token_kernel(dirs):
+    """The same whole prompts with the matrix-core kernel switched off: both kernels round differently, no more."""
+    from mini_llm_amd.kernels import ops
+    cfg, d = kc.TILED, dirs("TILED")
+    reqs = kc.requests(cfg["vocab"], [5, 100, 257], seed=72)
+    steps = ru.trace_whole(reqs)
+    got = []
+    try:
+        for on in (True, False):
+            ops.set_latent_tiles(on)
+            ops.reset_seen()
+            runner = _runner(d, "bfloat16", n_pages=ru.peak_tokens(steps) // 16, page=16)
+            got.append(ru.collect(steps, ru.run_in_process(runner, steps), cfg["vocab"]))
+            assert (ops.seen("latent_tile_launches") > 0) == on
+    finally:
+        ops.set_latent_tiles(True)
+    worst = max(kc.row_error(got[0][r][p], got[1][r][p].astype(np.float64)) for r in reqs for p in range(len(reqs[r])))
+    print(f"matrix-core kernel against the per-token kernel: {worst:.3e}")
+    assert worst <= 2e-2
+
+
 @pytest.mark.parametrize("page", [2, 4, 16])
 def test_window_and_page_borders_with_peaked_scores(dirs, page):
     """Scores scaled so that single keys dominate, windows of 5, 6 and 16 over pages of 2, 4 and 16 tokens: a
