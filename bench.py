@@ -32,6 +32,35 @@ def small_config(n_layer, size="gpt2-small", n_positions=1024):
                 activation_function="gelu_new", eos_token_id=50256, bos_token_id=50256)
 
 
+def kugulorn_config(n_layer, size="gpt2-small", n_positions=1024):
+    """A Kugulorn model of about the size of the GPT-2 configuration `size`: the same width, number of layers,
+    vocabulary and context; Mamba-2 layers (inner width twice the model's, heads of 64, a state of 128 rows) and
+    latent-attention layers (as many heads as GPT-2 has, a latent of a third of the width beside 32 rotated
+    columns, every second one reading the pages of the one before it, the window as long as the context) in
+    turn, each with a gated feed-forward whose three matrices hold what GPT-2's two do."""
+    full_layers, d, h, f = SIZES[size]
+    n = n_layer or full_layers
+    rank = max(64, d // 3 // 32 * 32)                    # 256 at 768, 320 at 1024, 512 at 1600
+    ff = f * 2 // 3 // 64 * 64
+    mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+    layers, last_own = [], None
+    for i in range(n):
+        if i % 2 == 0:
+            layers.append({"type": "mamba2", "mlp": mlp,
+                           "mixer": {"heads": 2 * d // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}})
+        else:
+            m = {"heads": h, "dim": 64, "rot_dim": 32, "vdim": 64, "kv_rank": rank, "q_rank": d // 2, "scale": 96 ** -0.5,
+                 "mask": {"size": n_positions}, "rot": {"base": 10000.0, "dims": 32}}
+            if last_own is not None and (i // 2) % 2 == 1:
+                m["kv_from"] = last_own
+            else:
+                last_own = i
+            layers.append({"type": "latent_attention", "mixer": m, "mlp": mlp})
+    return {"architecture": "Kugulorn", "vocab": 50257, "width": d, "residual_mult": 1.0, "norm": {"eps": 1e-6}, "layers": layers,
+            # (what the measurement itself reads; the architecture ignores them)
+            "vocab_size": 50257, "n_positions": n_positions, "n_layer": n}
+
+
 def decode_run(model_dir, dtype, batch, prompt_len, steps, warmup, cfg):
     """Decode steps of `batch` requests through the whole engine. Every prompt is fed in ONE step before
     the clock starts, so that all requests decode in lockstep from position prompt_len on. Returns
@@ -75,7 +104,8 @@ def decode_run(model_dir, dtype, batch, prompt_len, steps, warmup, cfg):
     assert n_tok == batch * steps, (n_tok, batch, steps)
     mean_ctx = ctx0 + (steps - 1) / 2.0
     info = engine.runner.info()
-    bytes_step = info["weight_bytes"] + batch * mean_ctx * info["cache_bytes_per_token"]
+    # (a request's recurrent state, where the model has one, is read and written once a step)
+    bytes_step = info["weight_bytes"] + batch * (mean_ctx * info["cache_bytes_per_token"] + 2 * info.get("state_bytes_per_request", 0))
     per_step.sort()
     p50 = per_step[len(per_step) // 2]
     engine.close()
@@ -205,6 +235,36 @@ def serving_main(args, cfg, model_dir):
     return 0
 
 
+def compare_main(args):
+    """--compare: both designs at one size through prefill_run and decode_run."""
+    from mini_llm_amd import Runner, write_random_model
+    out = {"metric": f"Kugulorn beside GPT-2 at {args.size} sizes: prefill tok/s (2 x 1,024 tokens) and decode tok/s",
+           "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights seed 2, uniform random token ids)",
+           "n_gpus": 1, "designs": {}}
+    for design in ("gpt2", "kugulorn"):
+        cfg = (kugulorn_config if design == "kugulorn" else small_config)(args.layers, args.size, args.positions)
+        with tempfile.TemporaryDirectory() as d:
+            write_random_model(dict(cfg), d, seed=2)
+            r = Runner(model_dir=d, dtype=args.dtype, page_size=16, n_pages=8, max_num_seqs=1)
+            info = r.info()
+            del r
+            ptps, pdt, flops = prefill_run(d, args.dtype, cfg)
+            rec = {"n_layer": cfg["n_layer"], "weight_bytes": int(info["weight_bytes"]), "cache_bytes_per_token": info["cache_bytes_per_token"],
+                   "state_bytes_per_request": info.get("state_bytes_per_request", 0),
+                   "prefill": {"tok_per_s": round(ptps, 1), "ms": round(pdt * 1e3, 4), "tflops": round(flops / pdt / 1e12, 1),
+                               "frac_of_peak": round(flops / pdt / MFMA_PEAK[args.dtype], 5)}}
+            for b in (1, 8, 64):
+                tps, step_s, p50, mean_ctx, bytes_step = decode_run(d, args.dtype, b, args.prompt_len, min(args.steps, 128), min(args.warmup, 16), cfg)
+                rec[f"decode_b{b}"] = {"tok_per_s": round(tps, 1), "ms_per_step": round(step_s * 1e3, 4), "mean_context": round(mean_ctx, 1),
+                                       "GBps": round(bytes_step / step_s / 1e9, 1), "frac_of_hbm_peak": round(bytes_step / step_s / HBM_PEAK, 5)}
+            out["designs"][design] = rec
+    g, k = out["designs"]["gpt2"], out["designs"]["kugulorn"]
+    out["kugulorn_over_gpt2"] = {"prefill": round(k["prefill"]["tok_per_s"] / g["prefill"]["tok_per_s"], 3),
+                                 **{f"decode_b{b}": round(k[f"decode_b{b}"]["tok_per_s"] / g[f"decode_b{b}"]["tok_per_s"], 3) for b in (1, 8, 64)}}
+    print(json.dumps(out))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -229,6 +289,12 @@ def main():
     ap.add_argument("--config", help="a config.json to measure in place of the GPT-2 sizes (any registered architecture; "
                                      "it names vocab_size and n_positions, or --vocab / --positions do)")
     ap.add_argument("--vocab", type=int, default=0, help="with --config: the vocabulary to draw token ids from")
+    ap.add_argument("--design", default="gpt2", choices=["gpt2", "kugulorn"],
+                    help="kugulorn: a Kugulorn model of about the size --size names (kugulorn_config) through the same "
+                         "measurement; --compare runs both designs one after the other")
+    ap.add_argument("--compare", action="store_true",
+                    help="prefill (2 x 1,024 tokens) and decode (batch 1, 8, 64) of the Kugulorn model and of the GPT-2 model "
+                         "of --size, side by side in one JSON line")
     ap.add_argument("--peaks-only", action="store_true",
                     help="measure this GPU's streaming bandwidth and matrix-core rate and print them")
     ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "kv-pressure"],
@@ -243,6 +309,10 @@ def main():
     for path in args.plugin:
         load_plugin(path)
     cfg = small_config(args.layers, args.size, args.positions)
+    if args.compare:
+        return compare_main(args)
+    if args.design == "kugulorn":
+        cfg = kugulorn_config(args.layers, args.size, args.positions)
     if args.config:
         # another architecture, served by the same engine: sizes from its own config.json
         with open(args.config) as f:
@@ -255,7 +325,7 @@ def main():
             print("bench.py: --config names no vocab_size; give --vocab")
             return 2
         cfg.setdefault("n_layer", None)
-        args.size = cfg.get("architectures", ["?"])[0]
+        args.size = cfg.get("architectures", [cfg.get("architecture", "?")])[0]
         SIZES[args.size] = (cfg["n_layer"], 0, 0, 0)
     if "n_embd" not in cfg:
         args.no_points = True
@@ -296,7 +366,8 @@ def main():
             "higher_is_better": True, "scaling": "weak",
             "vs_baseline": round(tps / reference_tps, 2) if reference_tps else None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic (random weights seed 2, uniform random token ids)",
-            "config": {"model": args.size + "-sizes", "n_layer": cfg["n_layer"], "n_layer_full": SIZES[args.size][0],
+            "config": {"model": args.size + "-sizes" + (" (Kugulorn)" if args.design == "kugulorn" else ""),
+                       "n_layer": cfg["n_layer"], "n_layer_full": SIZES[args.size][0],
                        "n_embd": cfg.get("n_embd"), "n_head": cfg.get("n_head"),
                        "head_dim": cfg["n_embd"] // cfg["n_head"] if "n_embd" in cfg else None,
                        "n_inner": cfg.get("n_inner"), "vocab_size": cfg["vocab_size"],

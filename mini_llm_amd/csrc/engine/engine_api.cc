@@ -325,7 +325,7 @@ int mllm_runner_check(void* runner, char* out, int cap) {
     return put_text(text, out, cap);
 }
 // Sizes and costs as JSON: architecture, vocab_size, hidden_size, max_positions, eos_token_id, dtype, n_layers,
-// n_calls, n_caches, n_groups, page_size, n_pages, free_pages, n_requests, cache_bytes_per_token, and the step's
+// n_calls, n_caches, n_groups, page_size, n_pages, free_pages, n_requests, cache_bytes_per_token, state_bytes_per_request, and the step's
 // cost (parts.h: StepCost): weight_bytes, flops_per_token, attention_flops_per_key, flops_per_logits_row
 int mllm_runner_info(void* runner, char* out, int cap) {
     std::string text;
@@ -349,6 +349,9 @@ int mllm_runner_info(void* runner, char* out, int cap) {
         j.set("free_pages", Json::of(r->manager().n_groups() ? r->manager().free_pages(0) : 0));
         j.set("n_requests", Json::of(r->manager().n_requests()));
         j.set("cache_bytes_per_token", Json::of(static_cast<int64_t>(r->cache().bytes_per_token())));
+        int64_t state_bytes = 0;
+        for (const CacheNeed& n : m.caches) if (n.kind == 2) state_bytes += static_cast<int64_t>(n.state_bytes);
+        j.set("state_bytes_per_request", Json::of(state_bytes));
         j.set("weight_bytes", Json::of(c.weight_bytes));
         j.set("flops_per_token", Json::of(c.flops_per_token));
         j.set("attention_flops_per_key", Json::of(c.attention_flops_per_key));

@@ -94,7 +94,11 @@ public:
         LatentStep ls;
         ls.block_tables = step.block_tables[g]; ls.max_blocks = step.max_blocks[g]; ls.n_seqs = step.n_seqs; ls.max_q_len = step.max_q_len;
         ls.token_seq = step.token_seq; ls.positions = step.positions; ls.cu_q = step.cu_q; ls.ctx_len = step.ctx_len;
-        latent_attention(qa, pages, ls, scale_, window_, sh_, o_lat, s);
+        ls.max_ctx_len = step.max_ctx_len;
+        // (room for the states of split keys, used by steps of few rows only)
+        const size_t ws_floats = dtype_ == BF16 ? latent_attention_workspace_floats(sh_.kv_rank) : 0;
+        float* ws = ws_floats ? static_cast<float*>(arena.take(ws_floats * 4)) : nullptr;
+        latent_attention(qa, pages, ls, scale_, window_, sh_, o_lat, ws, ws_floats, s);
         StageTimes::get().mark("attention", s);
         Tensor2 o = arena.tensor(dtype_, T, H * sh_.value_dim);
         latent_expand(o_lat, uv_, o, sh_, s);
@@ -104,7 +108,7 @@ public:
     size_t workspace_bytes(int tokens) const override {
         const size_t E = sh_.kv_rank + sh_.rot_dim, H = sh_.n_heads;
         const size_t per_token = (sh_.q_rank + E) * 4 + (dq_.in_features() + sh_.q_rank + H * (sh_.plain_dim + sh_.rot_dim) + H * E + H * sh_.kv_rank + H * sh_.value_dim) * dtype_size(dtype_);
-        return static_cast<size_t>(tokens) * per_token + 4096;
+        return static_cast<size_t>(tokens) * per_token + (dtype_ == BF16 ? latent_attention_workspace_floats(sh_.kv_rank) * 4 : 0) + 8192;
     }
     CacheNeed cache_need() const override {
         CacheNeed n;

@@ -59,11 +59,15 @@ public:
         StateArgs st;
         st.token_seq = step.token_seq; st.cu_q = step.cu_q; st.state_slots = step.state_slots; st.n_seqs = step.n_seqs;
         st.state = static_cast<float*>(cache.state); st.slot_floats = slot_floats_; st.n_slots = cache.n_slots; st.write = write;
+        st.max_q_len = step.max_q_len;
         Tensor2 xbc = arena.tensor(F32, T, channels_);
         conv_silu(proj, inner_, conv_, conv_bias_, st, xbc, s);
         StageTimes::get().mark("conv", s);
         Tensor2 y = arena.tensor(F32, T, inner_);
-        ssm_scan(xbc, proj, 2 * inner_ + 2 * G_ * N_, dt_bias_, A_log_, D_, st, carried_floats_, H_, P_, N_, G_, y, s);
+        // (portions longer than a chunk are scanned chunk by chunk side by side: room for the chunks' states)
+        const size_t ws_floats = step.max_q_len > 64 ? ssm_scan_workspace_floats(T, step.n_seqs, H_, P_, N_) : 0;
+        float* ws = ws_floats ? static_cast<float*>(arena.take(ws_floats * 4)) : nullptr;
+        ssm_scan(xbc, proj, 2 * inner_ + 2 * G_ * N_, dt_bias_, A_log_, D_, st, carried_floats_, H_, P_, N_, G_, y, ws, ws_floats, s);
         StageTimes::get().mark("scan", s);
         Tensor2 gated = arena.tensor(dtype_, T, inner_);
         const Tensor2 z(proj.data, F32, T, inner_, proj.stride);
@@ -72,7 +76,8 @@ public:
         StageTimes::get().mark("out_proj", s);
     }
     size_t workspace_bytes(int tokens) const override {
-        return static_cast<size_t>(tokens) * ((in_.out_features() + 4) * 4 + channels_ * 4 + inner_ * 4 + inner_ * dtype_size(dtype_)) + 4096;
+        return static_cast<size_t>(tokens) * ((in_.out_features() + 4) * 4 + channels_ * 4 + inner_ * 4 + inner_ * dtype_size(dtype_)) +
+               ssm_scan_workspace_floats(tokens, 1, H_, P_, N_) * 4 + 8192;
     }
     CacheNeed cache_need() const override {
         CacheNeed n;

@@ -172,7 +172,7 @@ struct StateArgs {
     const int* token_seq = nullptr;    // [T]
     const int* cu_q = nullptr;         // [B + 1]
     const int* state_slots = nullptr;  // [B], < 0: padding
-    int n_seqs = 0;
+    int n_seqs = 0, max_q_len = 0;     // max_q_len: the longest portion of the step
     float* state = nullptr;
     size_t slot_floats = 0;
     int n_slots = 0;
@@ -183,10 +183,12 @@ struct StateArgs {
 void conv_silu(const Tensor2& proj, int col0, const Tensor2& weight, const float* bias, const StateArgs& st,
                const Tensor2& out, hipStream_t stream);
 // The Mamba-2 scan (kernels/ssm.hip) over xbc [T, H*P + 2*G*N] and the raw step sizes (columns dt_col.. of
-// proj), state at `scan_offset` floats into the slot; y [T, H*P] fp32.
+// proj), state at `scan_offset` floats into the slot; y [T, H*P] fp32. Portions longer than a chunk are
+// scanned chunk by chunk side by side and joined, for which `workspace` (ssm_scan_workspace_floats floats) is needed.
 void ssm_scan(const Tensor2& xbc, const Tensor2& proj, int dt_col, const float* dt_bias, const float* A_log,
               const float* skip, const StateArgs& st, size_t scan_offset, int H, int P, int N, int G, const Tensor2& y,
-              hipStream_t stream);
+              float* workspace, size_t workspace_floats, hipStream_t stream);
+size_t ssm_scan_workspace_floats(int tokens, int n_seqs, int H, int P, int N);
 
 // -- latent attention --------------------------------------------------------------------------------
 struct LatentShape {
@@ -210,17 +212,19 @@ void latent_absorb(const Tensor2& q, const Tensor2& w_uk, const Tensor2& qa, con
 // The step's sequences, as attention sees them.
 struct LatentStep {
     const int* block_tables = nullptr;     // [n_seqs, max_blocks]
-    int max_blocks = 0, n_seqs = 0, max_q_len = 0;
+    int max_blocks = 0, n_seqs = 0, max_q_len = 0, max_ctx_len = 0;
     const int* token_seq = nullptr;        // [T]
     const int* positions = nullptr;        // [T]
     const int* cu_q = nullptr;             // [n_seqs + 1]
     const int* ctx_len = nullptr;          // [n_seqs]
 };
 // o_lat[t, h] = sum_j softmax_j(scale * qa[t, h] . row_j) row_j[:kv_rank] over the visible rows of the pages.
-// Steps with prompt portions run on the matrix cores where the sizes allow (bfloat16, the transposed latent
-// at hand), others one workgroup per token.
+// Runs on the matrix cores where the sizes allow (bfloat16, the transposed latent at hand), otherwise one
+// workgroup per token. `workspace` (optional, fp32, latent_attention_workspace_floats(...) floats): steps of few
+// rows (decoding) then spread every row's keys over several workgroups, whose states meet there.
 void latent_attention(const Tensor2& qa, const LatentPages& pages, const LatentStep& step, float scale, int window,
-                      const LatentShape& sh, const Tensor2& o_lat, hipStream_t stream);
+                      const LatentShape& sh, const Tensor2& o_lat, float* workspace, size_t workspace_floats, hipStream_t stream);
+size_t latent_attention_workspace_floats(int kv_rank);
 // out[t, h*value_dim + e] = sum_r w_uv[h*value_dim + e, r] * o_lat[t, h, r]
 void latent_expand(const Tensor2& o_lat, const Tensor2& w_uv, const Tensor2& out, const LatentShape& sh, hipStream_t stream);
 

@@ -94,7 +94,7 @@ void conv_silu(const Tensor2& proj, int col0, const Tensor2& weight, const float
 
 void ssm_scan(const Tensor2& xbc, const Tensor2& proj, int dt_col, const float* dt_bias, const float* A_log,
               const float* skip, const StateArgs& st, size_t scan_offset, int H, int P, int N, int G, const Tensor2& y,
-              hipStream_t stream) {
+              float* workspace, size_t workspace_floats, hipStream_t stream) {
     need_f32(xbc, "ssm_scan: x, B, C");
     need_f32(proj, "ssm_scan: the step sizes");
     need_f32(y, "ssm_scan: y");
@@ -105,9 +105,18 @@ void ssm_scan(const Tensor2& xbc, const Tensor2& proj, int dt_col, const float* 
     if (y.rows != xbc.rows || y.cols != static_cast<int64_t>(H) * P) fail("ssm_scan: y must be [%lld, %d]", (long long)xbc.rows, H * P);
     if (dt_bias == nullptr || A_log == nullptr || skip == nullptr) fail("ssm_scan: dt_bias, A_log and D are needed");
     check_state(st, scan_offset + static_cast<size_t>(H) * P * N, "ssm_scan");
+    const int T = i32(xbc.rows);
+    // (a step whose longest portion is unknown is taken to have a long one)
+    const int max_q = st.max_q_len > 0 ? st.max_q_len : T;
+    if (workspace != nullptr && workspace_floats < ssm_scan_workspace_floats(T, st.n_seqs, H, P, N))
+        fail("ssm_scan: the workspace holds %zu floats, %zu are needed", workspace_floats, ssm_scan_workspace_floats(T, st.n_seqs, H, P, N));
     check(mllm_ssm_scan(static_cast<const float*>(xbc.data), i32(xbc.stride), static_cast<const float*>(proj.data) + dt_col, i32(proj.stride),
                         dt_bias, A_log, skip, st.cu_q, st.state_slots, st.state, st.slot_floats, scan_offset, static_cast<float*>(y.data),
-                        i32(y.stride), st.n_seqs, H, P, N, G, st.write ? 1 : 0, stream), "ssm_scan");
+                        i32(y.stride), T, st.n_seqs, max_q, H, P, N, G, st.write ? 1 : 0, workspace, stream), "ssm_scan");
+}
+
+size_t ssm_scan_workspace_floats(int tokens, int n_seqs, int H, int P, int N) {
+    return mllm_ssm_scan_workspace_floats(tokens, n_seqs, H, P, N);
 }
 
 static void check_shape(const LatentShape& sh, const char* what) {
@@ -161,8 +170,12 @@ void latent_absorb(const Tensor2& q, const Tensor2& w_uk, const Tensor2& qa, con
                              sh.plain_dim, sh.rot_dim, sh.kv_rank, sh.rot_base, sh.rot_dims, q.dtype, stream), "latent_absorb");
 }
 
+// Rows x splits that a launch with split keys holds at most (its workspace is made for them).
+constexpr long long LATENT_SPLIT_ROWS = 512 * 64;
+size_t latent_attention_workspace_floats(int kv_rank) { return static_cast<size_t>(LATENT_SPLIT_ROWS) * (kv_rank + 2); }
+
 void latent_attention(const Tensor2& qa, const LatentPages& pages, const LatentStep& step, float scale, int window,
-                      const LatentShape& sh, const Tensor2& o_lat, hipStream_t stream) {
+                      const LatentShape& sh, const Tensor2& o_lat, float* workspace, size_t workspace_floats, hipStream_t stream) {
     check_shape(sh, "latent_attention");
     need_act(qa, "latent_attention: qa");
     const int E = sh.kv_rank + sh.rot_dim, T = i32(qa.rows);
@@ -174,14 +187,22 @@ void latent_attention(const Tensor2& qa, const LatentPages& pages, const LatentS
         fail("latent_attention: block tables, token_seq and positions are needed");
     if (qa.dtype == BF16 && E % 2 != 0) fail("latent_attention: rows of %d bfloat16 columns are not supported (an even number is)", E);
     if (window < 0) fail("latent_attention: a negative window");
-    // prompt portions: the matrix-core kernel, one workgroup per 64 (token, head) rows of a sequence
-    if (tuning().latent_tiles && step.max_q_len > 1 && qa.dtype == BF16 && pages.latent_t.data != nullptr && step.cu_q != nullptr &&
+    // the matrix-core kernel: one workgroup per 64 (token, head) rows of a sequence
+    if (tuning().latent_tiles && qa.dtype == BF16 && pages.latent_t.data != nullptr && step.cu_q != nullptr &&
         step.ctx_len != nullptr && step.n_seqs > 0 && qa.contiguous() && o_lat.contiguous()) {
-        const long long tiles = static_cast<long long>(T) * sh.n_heads / 64 + step.n_seqs;
+        const long long rows = static_cast<long long>(T) * sh.n_heads, tiles = rows / 64 + step.n_seqs;
         if (tiles < (1ll << 31)) {
+            // Few workgroups (decoding): every row's key tiles are spread over several, so that about 512
+            // workgroups stream the pages instead of one per sequence walking its tiles one after the other.
+            const int keys = window > 0 ? std::min(window, std::max(step.max_ctx_len, 1)) : std::max(step.max_ctx_len, 1);
+            int nsplit = 1;
+            if (workspace != nullptr && tiles < 256) {
+                nsplit = static_cast<int>(std::min<long long>({(keys + 63) / 64 + 1, 512 / tiles, LATENT_SPLIT_ROWS / std::max<long long>(rows, 1)}));
+                if (nsplit < 2 || static_cast<size_t>(rows) * nsplit * (sh.kv_rank + 2) > workspace_floats) nsplit = 1;
+            }
             const int rc = mllm_latent_attention_tiles(qa.data, pages.rows.data, pages.latent_t.data, step.block_tables, step.max_blocks, step.cu_q,
                                                        step.ctx_len, step.n_seqs, static_cast<int>(tiles), sh.n_heads, sh.kv_rank, sh.rot_dim,
-                                                       pages.page_size, scale, window, o_lat.data, stream);
+                                                       pages.page_size, scale, window, o_lat.data, static_cast<int>(rows), nsplit, workspace, stream);
             if (rc == 0) { tuning().seen.latent_tile_launches += 1; return; }
             if (rc != -2) check(rc, "latent_attention (tiles)");
         }

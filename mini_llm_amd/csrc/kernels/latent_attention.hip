@@ -252,7 +252,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))
 latent_prefill_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
                       const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
                       const int* __restrict__ ctx_len, int n_seqs, int H, int page_size, float scale_log2e, int window,
-                      bf16_t* __restrict__ o_lat) {
+                      bf16_t* __restrict__ o_lat, int nsplit, float* __restrict__ partials) {
     constexpr int E = 32 * KS, R = 16 * DT, BN = 64, KSTRIDE = E + 8, VSTRIDE = BN + 8, CH = E / 8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     bf16_t* Ks = reinterpret_cast<bf16_t*>(smem);                    // [BN][KSTRIDE]
@@ -294,7 +294,15 @@ latent_prefill_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ 
     for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int pg_lo = k_lo >> shift, pg_hi = p_last >> shift;
 
-    for (int kt = k_lo / BN; kt <= p_last / BN; ++kt) {
+    // With nsplit > 1 (few rows in the step: decoding) the workgroups blockIdx.y = 0 .. nsplit - 1 share the
+    // key tiles of these rows and leave their states unmerged in `partials`.
+    int kt_begin = k_lo / BN, kt_end = p_last / BN + 1;
+    if (nsplit > 1) {
+        const int per = (kt_end - kt_begin + nsplit - 1) / nsplit;
+        kt_begin += static_cast<int>(blockIdx.y) * per;
+        kt_end = min(kt_end, kt_begin + per);
+    }
+    for (int kt = kt_begin; kt < kt_end; ++kt) {
         const int j_base = kt * BN;
         __syncthreads();                           // the tile before is used up
         // page rows, row-major; a key outside [k_lo, p_last] is replaced by one inside (always a held page;
@@ -382,6 +390,17 @@ latent_prefill_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ 
     }
     l = rows_sum(l);
     if (!q_ok) return;
+    if (nsplit > 1) {
+        // this split's state of the row: [maximum (base 2, scaled), sum, unnormalised output]; a split that saw
+        // no key leaves maximum -inf, sum 0, zeros
+        float* st = partials + ((static_cast<size_t>(q_begin) * H + rho) * nsplit + blockIdx.y) * (R + 2);
+        if (G == 0) { st[0] = m; st[1] = l; }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) st[2 + 16 * dt + 4 * G + r] = o[dt][r];
+        return;
+    }
     const float inv = 1.0f / l;
     // o[dt][r] is latent column 16 dt + 4 G + r of this lane's query row
     bf16_t* orow = o_lat + (static_cast<size_t>(q_begin) * H + rho) * R;
@@ -391,6 +410,28 @@ latent_prefill_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ 
         pk.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
         pk.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
         *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * G) = pk;
+    }
+}
+
+// The splits' states of a row merged: o = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s. One wavefront per row.
+__global__ void __launch_bounds__(256)
+latent_merge_kernel(const float* __restrict__ partials, int n_rows, int nsplit, int R, bf16_t* __restrict__ o_lat) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
+    const int row = blockIdx.x * 4 + wave;
+    if (row >= n_rows) return;
+    const float* st = partials + static_cast<size_t>(row) * nsplit * (R + 2);
+    float M = -INFINITY;
+    for (int sp = 0; sp < nsplit; ++sp) M = fmaxf(M, st[static_cast<size_t>(sp) * (R + 2)]);
+    float L = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) L += fast_exp2(st[static_cast<size_t>(sp) * (R + 2)] - M) * st[static_cast<size_t>(sp) * (R + 2) + 1];
+    const float inv = 1.0f / L;
+    for (int c = lane; c < R; c += 64) {
+        float acc = 0.f;
+        for (int sp = 0; sp < nsplit; ++sp) {
+            const float* one = st + static_cast<size_t>(sp) * (R + 2);
+            acc += fast_exp2(one[0] - M) * one[2 + c];
+        }
+        o_lat[static_cast<size_t>(row) * R + c] = float_to_bf16(acc * inv);
     }
 }
 
@@ -479,16 +520,19 @@ int mllm_latent_attention(const void* qa, int ldqa, const void* pages, const int
     return 0;
 }
 
-// Prompt portions on the matrix cores (see latent_prefill_kernel): qa [T*H, E] and o_lat [T*H, R] contiguous
-// bfloat16. n_tiles_upper: an upper bound of sum over sequences of ceil(q_len * H / 64). Returns -2 when the
+// The matrix-core kernel (see latent_prefill_kernel): qa [T*H, E] and o_lat [T*H, R] contiguous bfloat16.
+// nsplit > 1: every row's key tiles are shared by nsplit workgroups whose states meet in `partials`
+// (n_rows * nsplit * (R + 2) floats, n_rows = T*H) and are merged by a second kernel. n_tiles_upper: an upper bound of sum over sequences of ceil(q_len * H / 64). Returns -2 when the
 // sizes are not ones it is built for (E and R among (128, 96), (96, 64), (160, 128), (288, 256), (576, 512);
 // page sizes 8 to 64, powers of two; a block table that fits the LDS beside the tiles): the caller then runs
 // mllm_latent_attention.
 int mllm_latent_attention_tiles(const void* qa, const void* k_pages, const void* vt_pages, const int* block_tables,
                                 int max_blocks, const int* cu_q, const int* ctx_len, int n_seqs, int n_tiles_upper, int H,
-                                int R, int Dr, int page_size, float scale, int window, void* o_lat, hipStream_t stream) {
+                                int R, int Dr, int page_size, float scale, int window, void* o_lat, int n_rows, int nsplit,
+                                float* partials, hipStream_t stream) {
     if (n_seqs <= 0 || n_tiles_upper <= 0) return 0;
     const int E = R + Dr;
+    if (nsplit < 1 || nsplit > 65535 || (nsplit > 1 && (partials == nullptr || n_rows < 1))) return -1;
     if (E % 32 != 0 || R % 16 != 0 || page_size < 8 || page_size > 64 || (page_size & (page_size - 1)) != 0) return -2;
     if (((reinterpret_cast<uintptr_t>(qa) | reinterpret_cast<uintptr_t>(k_pages) | reinterpret_cast<uintptr_t>(vt_pages) |
           reinterpret_cast<uintptr_t>(o_lat)) & 15) != 0)
@@ -505,10 +549,16 @@ int mllm_latent_attention_tiles(const void* qa, const void* k_pages, const void*
             if (e != hipSuccess) return static_cast<int>(e);                                                         \
             allowed = true;                                                                                          \
         }                                                                                                            \
-        latent_prefill_kernel<KS, DT><<<n_tiles_upper, 256, lds, stream>>>(                                          \
+        latent_prefill_kernel<KS, DT><<<dim3(n_tiles_upper, nsplit), 256, lds, stream>>>(                            \
             static_cast<const bf16_t*>(qa), static_cast<const bf16_t*>(k_pages), static_cast<const bf16_t*>(vt_pages), \
-            block_tables, max_blocks, cu_q, ctx_len, n_seqs, H, page_size, sl2, window, static_cast<bf16_t*>(o_lat)); \
+            block_tables, max_blocks, cu_q, ctx_len, n_seqs, H, page_size, sl2, window, static_cast<bf16_t*>(o_lat), \
+            nsplit, partials);                                                                                       \
         MLLM_LAUNCH_CHECK();                                                                                         \
+        if (nsplit > 1) {                                                                                            \
+            latent_merge_kernel<<<(n_rows + 3) / 4, 256, 0, stream>>>(partials, n_rows, nsplit, R,                   \
+                                                                     static_cast<bf16_t*>(o_lat));                  \
+            MLLM_LAUNCH_CHECK();                                                                                     \
+        }                                                                                                            \
         return 0;                                                                                                    \
     }
     LP_CASE(4, 6) LP_CASE(3, 4) LP_CASE(5, 8) LP_CASE(9, 16) LP_CASE(18, 32)

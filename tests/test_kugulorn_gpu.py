@@ -45,8 +45,10 @@ def _families(reqs, seed):
 @pytest.mark.parametrize("name", ["ONLY_MAMBA", "ONLY_MAMBA_WIDE_STATE", "ONLY_LATENT", "ONLY_LATENT_MLP"])
 def test_each_mechanism_alone(dirs, name, dtype):
     cfg, d = getattr(kc, name), dirs(name)
-    reqs = kc.requests(cfg["vocab"], [1, 2, 3, 9, 37], seed=5)
-    for label, steps in (("whole", ru.trace_whole(reqs)), ("chunks", ru.trace_chunks(reqs, seed=1))):
+    # (portions of more than 64 tokens: the scan cuts them into chunks that run side by side)
+    reqs = kc.requests(cfg["vocab"], [1, 2, 3, 9, 37, 64, 65, 200], seed=5)
+    for label, steps in (("whole", ru.trace_whole(reqs)), ("chunks", ru.trace_chunks(reqs, seed=1)),
+                         ("long chunks", ru.trace_chunks(reqs, seed=1, sizes=(70, 3, 129)))):
         runner = _runner(d, dtype, n_pages=ru.peak_tokens(steps) // 4)
         kc.check_against_plain(d, reqs, steps, ru.run_in_process(runner, steps), dtype, cfg["vocab"], f"{name} {label}")
         assert runner.check() == "" and runner.info()["n_requests"] == 0
