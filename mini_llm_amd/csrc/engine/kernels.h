@@ -60,7 +60,7 @@ int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const vo
 
 // norm_gate.hip
 int mllm_rmsnorm(const float* x, int ldx, const int* rows, const float* w, const float* gate, int ldg, void* y, int ldy,
-                 int n, int D, int groups, float eps, int out_dtype, hipStream_t stream);
+                 int n, int D, int groups, float eps, int out_dtype, int parts, size_t part_stride, hipStream_t stream);
 int mllm_rmsnorm_add(float* y, const float* w, const float* scale, float mult, float eps, float* x, int n, int D,
                      int clear, hipStream_t stream);
 int mllm_glu_clamped(const void* gate, int ldg, const void* up, int ldu, void* out, int ldo, int T, int F, float limit,
@@ -73,8 +73,9 @@ int mllm_conv_silu(const float* proj, int ld, int col0, int C, const float* w, c
                    float* out, int ldo, int T, int B, int write, hipStream_t stream);
 int mllm_ssm_scan(const float* xbc, int ldx, const float* raw_dt, int ldd, const float* dt_bias, const float* A_log,
                   const float* Dskip, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
-                  size_t scan_offset, float* y, int ldy, int T, int B, int max_q_len, int H, int P, int N, int G, int write,
-                  float* workspace, hipStream_t stream);
+                  size_t scan_offset, float* y, int ldy, size_t part_stride, int T, int B, int max_q_len, int H, int P, int N,
+                  int G, int write, float* workspace, hipStream_t stream);
+int mllm_ssm_scan_parts(int N);
 size_t mllm_ssm_scan_workspace_floats(int T, int B, int H, int P, int N);
 
 // latent_attention.hip
@@ -89,7 +90,7 @@ int mllm_latent_attention(const void* qa, int ldqa, const void* pages, const int
 int mllm_latent_attention_tiles(const void* qa, const void* k_pages, const void* vt_pages, const int* block_tables,
                                 int max_blocks, const int* cu_q, const int* ctx_len, int n_seqs, int n_tiles_upper, int H,
                                 int R, int Dr, int page_size, float scale, int window, void* o_lat, int n_rows, int nsplit,
-                                float* partials, hipStream_t stream);
+                                float* partials, int single_tokens, hipStream_t stream);
 int mllm_latent_expand(const void* o_lat, int ldo, const void* w_uv, int ldw, void* out, int ldout, int T, int H, int Dv, int R,
                        int dtype, hipStream_t stream);
 

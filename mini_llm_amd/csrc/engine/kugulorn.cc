@@ -79,7 +79,6 @@ struct KugulornConfig {
                 if (lc.heads % lc.groups != 0) throw ConfigError("config.json: " + where + "heads is not a multiple of groups");
                 if ((lc.heads * lc.vdim) % lc.norm_groups != 0) throw ConfigError("config.json: " + where + "heads * vdim is not a multiple of norm_groups");
                 if (lc.conv > 16) throw ConfigError("config.json: " + where + "a convolution of more than 16 taps is not supported");
-                if (lc.state > 1024) throw ConfigError("config.json: " + where + "a state of more than 1024 rows is not supported");
             } else if (type->string() == "latent_attention") {
                 lc.kind = LayerConfig::LatentAttention;
                 lc.heads = need_int(m, "heads", where); lc.dim = need_int(m, "dim", where); lc.rot_dim = need_int(m, "rot_dim", where, 0);
@@ -156,7 +155,8 @@ std::vector<ParamSpec> kugulorn_specs(const Json& config) {
                 matrix(M + "dkv", l.kv_rank + l.rot_dim, D);
                 vector(M + "dkv.norm", l.kv_rank, 1.0, 0.1);
             }
-            matrix(M + "uk", l.heads * l.dim, l.kv_rank);
+            // (kept transposed, [kv_rank, heads * dim]: queries are multiplied by it, not the latent)
+            s.push_back({M + "uk", {l.heads * l.dim, l.kv_rank}, ParamSpec::Matrix, true, 0.0, 1.0 / std::sqrt(static_cast<double>(l.kv_rank))});
             matrix(M + "uv", l.heads * l.vdim, l.kv_rank);
             matrix(M + "o", D, l.heads * l.vdim);
         }

@@ -26,7 +26,8 @@ const float* f32_vector(const Params& p, const char* key, int n) {
 // The turn is the interleaved one: the pair (2i, 2i+1) of the first rot_dims rotated columns at position p
 // by the angle p * rot_base^(-2i / rot_dims).
 // Parameters: heads, plain_dim, rot_dim, value_dim, kv_rank, q_rank, window, scale, rot_base, rot_dims, eps,
-// dtype; tensors dq.weight, dq.norm, uq.weight, [dkv.weight, dkv.norm,] uk.weight, uv.weight, out.weight.
+// dtype; tensors dq.weight, dq.norm, uq.weight, [dkv.weight, dkv.norm,] uk.weight (transposed: [kv_rank,
+// heads * plain_dim], the layout in which queries are carried into the latent's space), uv.weight, out.weight.
 class LatentAttention final : public Mixer {
 public:
     explicit LatentAttention(const Params& p) {
@@ -55,7 +56,7 @@ public:
         uv_ = p.weights("uv.weight");
         if (dq_.out_features() != sh_.q_rank || uq_.in_features() != sh_.q_rank || uq_.out_features() != qd)
             fail("latent_attention: the query projections do not fit %d heads of %d + %d through %d", sh_.n_heads, sh_.plain_dim, sh_.rot_dim, sh_.q_rank);
-        if (uk_.rows != static_cast<int64_t>(sh_.n_heads) * sh_.plain_dim || uk_.cols != sh_.kv_rank || uv_.rows != static_cast<int64_t>(sh_.n_heads) * sh_.value_dim ||
+        if (uk_.cols != static_cast<int64_t>(sh_.n_heads) * sh_.plain_dim || uk_.rows != sh_.kv_rank || uv_.rows != static_cast<int64_t>(sh_.n_heads) * sh_.value_dim ||
             uv_.cols != sh_.kv_rank || uk_.dtype != dtype_ || uv_.dtype != dtype_)
             fail("latent_attention: the key/value expansions do not fit %d heads and a latent of %d", sh_.n_heads, sh_.kv_rank);
         if (out_.in_features() != sh_.n_heads * sh_.value_dim) fail("latent_attention: the out-projection does not take %d heads of %d", sh_.n_heads, sh_.value_dim);
@@ -121,8 +122,8 @@ public:
     void add_cost(StepCost& c) const override {
         dq_.add_cost(c); uq_.add_cost(c); out_.add_cost(c);
         if (own_kv_) dkv_.add_cost(c);
-        c.weight_bytes += static_cast<double>(uk_.rows + uv_.rows) * sh_.kv_rank * dtype_size(dtype_);
-        c.flops_per_token += 2.0 * (uk_.rows + uv_.rows) * sh_.kv_rank;
+        c.weight_bytes += static_cast<double>(uk_.cols + uv_.rows) * sh_.kv_rank * dtype_size(dtype_);
+        c.flops_per_token += 2.0 * (uk_.cols + uv_.rows) * sh_.kv_rank;
         c.attention_flops_per_key += 2.0 * sh_.n_heads * (2.0 * sh_.kv_rank + sh_.rot_dim);
     }
 

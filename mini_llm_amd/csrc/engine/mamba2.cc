@@ -28,7 +28,6 @@ public:
         eps_ = static_cast<float>(p.number("eps"));
         dtype_ = p.integer("dtype");
         if (H_ < 1 || P_ < 1 || N_ < 1 || G_ < 1 || H_ % G_ != 0) fail("mamba2: %d heads of %d, state %d, %d groups do not fit", H_, P_, N_, G_);
-        if (N_ > 1024) fail("mamba2: a state of %d rows is not supported (up to 1024)", N_);
         inner_ = H_ * P_;
         channels_ = inner_ + 2 * G_ * N_;
         if (norm_groups_ < 1 || inner_ % norm_groups_ != 0) fail("mamba2: %d columns do not split into %d norm groups", inner_, norm_groups_);
@@ -63,7 +62,9 @@ public:
         Tensor2 xbc = arena.tensor(F32, T, channels_);
         conv_silu(proj, inner_, conv_, conv_bias_, st, xbc, s);
         StageTimes::get().mark("conv", s);
-        Tensor2 y = arena.tensor(F32, T, inner_);
+        // (the scan leaves its result as shares, one per slice of the state's rows; the norm adds them)
+        const int parts = ssm_scan_parts(N_);
+        Tensor2 y(arena.take(static_cast<size_t>(parts) * T * inner_ * 4), F32, T, inner_);
         // (portions longer than a chunk are scanned chunk by chunk side by side: room for the chunks' states)
         const size_t ws_floats = step.max_q_len > 64 ? ssm_scan_workspace_floats(T, step.n_seqs, H_, P_, N_) : 0;
         float* ws = ws_floats ? static_cast<float*>(arena.take(ws_floats * 4)) : nullptr;
@@ -71,12 +72,12 @@ public:
         StageTimes::get().mark("scan", s);
         Tensor2 gated = arena.tensor(dtype_, T, inner_);
         const Tensor2 z(proj.data, F32, T, inner_, proj.stride);
-        rmsnorm(y, norm_, eps_, norm_groups_, &z, gated, nullptr, s);
+        rmsnorm(y, norm_, eps_, norm_groups_, &z, gated, nullptr, s, parts, static_cast<size_t>(T) * inner_);
         out_(gated, x, ADD_RESIDUAL, nullptr, s);
         StageTimes::get().mark("out_proj", s);
     }
     size_t workspace_bytes(int tokens) const override {
-        return static_cast<size_t>(tokens) * ((in_.out_features() + 4) * 4 + channels_ * 4 + inner_ * 4 + inner_ * dtype_size(dtype_)) +
+        return static_cast<size_t>(tokens) * ((in_.out_features() + 4) * 4 + channels_ * 4 + ssm_scan_parts(N_) * inner_ * 4 + inner_ * dtype_size(dtype_)) +
                ssm_scan_workspace_floats(tokens, 1, H_, P_, N_) * 4 + 8192;
     }
     CacheNeed cache_need() const override {

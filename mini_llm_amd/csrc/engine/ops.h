@@ -155,9 +155,10 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
 // -- RMS norms, gated activation ---------------------------------------------------------------------
 // out[i, :] = x[rows ? rows[i] : i, :] / sqrt(mean(.^2) + eps) * weight, the columns in `groups` equal parts
 // that are normed one by one; with `gate` (fp32, x's shape) the input is x * silu(gate) (the gate comes
-// before the norm). x fp32 (any row stride), out in its own dtype.
+// before the norm). x fp32 (any row stride), out in its own dtype. With parts > 1 the input is the sum of `parts`
+// arrays of x's shape that lie part_stride floats apart (x the first), added in the order of their index.
 void rmsnorm(const Tensor2& x, const float* weight, float eps, int groups, const Tensor2* gate, const Tensor2& out,
-             const int* rows, hipStream_t stream);
+             const int* rows, hipStream_t stream, int parts = 1, size_t part_stride = 0);
 // x += mult * scale * (y / sqrt(mean(y^2) + eps) * weight), row by row (scale: per column, or null);
 // `clear`: y is zero afterwards.
 void rmsnorm_add(const Tensor2& y, const float* weight, const float* scale, float mult, float eps, const Tensor2& x,
@@ -183,12 +184,15 @@ struct StateArgs {
 void conv_silu(const Tensor2& proj, int col0, const Tensor2& weight, const float* bias, const StateArgs& st,
                const Tensor2& out, hipStream_t stream);
 // The Mamba-2 scan (kernels/ssm.hip) over xbc [T, H*P + 2*G*N] and the raw step sizes (columns dt_col.. of
-// proj), state at `scan_offset` floats into the slot; y [T, H*P] fp32. Portions longer than a chunk are
-// scanned chunk by chunk side by side and joined, for which `workspace` (ssm_scan_workspace_floats floats) is needed.
+// proj), state at `scan_offset` floats into the slot. y comes as ssm_scan_parts(N) shares, each [T, H*P] fp32
+// and y.rows * y.stride floats after the one before (y is the first); their sum in the order of their index is
+// the result (rmsnorm adds them while it reads). Portions longer than a chunk are scanned chunk by chunk side by
+// side and joined, for which `workspace` (ssm_scan_workspace_floats floats) is needed.
 void ssm_scan(const Tensor2& xbc, const Tensor2& proj, int dt_col, const float* dt_bias, const float* A_log,
               const float* skip, const StateArgs& st, size_t scan_offset, int H, int P, int N, int G, const Tensor2& y,
               float* workspace, size_t workspace_floats, hipStream_t stream);
 size_t ssm_scan_workspace_floats(int tokens, int n_seqs, int H, int P, int N);
+int ssm_scan_parts(int N);
 
 // -- latent attention --------------------------------------------------------------------------------
 struct LatentShape {
@@ -206,7 +210,7 @@ struct LatentPages {
 // cq = rmsnorm(dq) * wq; with dkv: page row slots[t] = [rmsnorm(dkv[:, :kv_rank]) * wkv | turned rest]
 void latent_prepare(const Tensor2& dq, const float* wq, const Tensor2& cq, const Tensor2* dkv, const float* wkv,
                     const LatentPages* pages, const int* slots, const int* positions, const LatentShape& sh, hipStream_t stream);
-// qa[t, h] = [W_uk_h^T q_plain[t, h] | turned q_rot[t, h]]
+// qa[t, h] = [W_uk_h^T q_plain[t, h] | turned q_rot[t, h]]; w_uk is handed over transposed, [kv_rank, heads * plain_dim]
 void latent_absorb(const Tensor2& q, const Tensor2& w_uk, const Tensor2& qa, const int* positions, const LatentShape& sh,
                    hipStream_t stream);
 // The step's sequences, as attention sees them.

@@ -31,7 +31,8 @@ void check_state(const StateArgs& st, size_t floats_needed, const char* what) {
 }  // namespace
 
 void rmsnorm(const Tensor2& x, const float* weight, float eps, int groups, const Tensor2* gate, const Tensor2& out,
-             const int* rows, hipStream_t stream) {
+             const int* rows, hipStream_t stream, int parts, size_t part_stride) {
+    if (parts < 1 || (parts > 1 && part_stride < static_cast<size_t>(x.rows) * x.stride)) fail("rmsnorm: %d parts %zu floats apart do not hold the input", parts, part_stride);
     need_f32(x, "rmsnorm: the input");
     need_act(out, "rmsnorm out");
     if (weight == nullptr) fail("rmsnorm: the weight is missing");
@@ -43,7 +44,8 @@ void rmsnorm(const Tensor2& x, const float* weight, float eps, int groups, const
         if (gate->rows != x.rows || gate->cols != x.cols) fail("rmsnorm: the gate must have the input's shape");
     }
     check(mllm_rmsnorm(static_cast<const float*>(x.data), i32(x.stride), rows, weight, gate ? static_cast<const float*>(gate->data) : nullptr,
-                       gate ? i32(gate->stride) : 0, out.data, i32(out.stride), i32(out.rows), i32(x.cols), groups, eps, out.dtype, stream),
+                       gate ? i32(gate->stride) : 0, out.data, i32(out.stride), i32(out.rows), i32(x.cols), groups, eps, out.dtype, parts,
+                       part_stride, stream),
           "rmsnorm");
 }
 
@@ -99,7 +101,6 @@ void ssm_scan(const Tensor2& xbc, const Tensor2& proj, int dt_col, const float* 
     need_f32(proj, "ssm_scan: the step sizes");
     need_f32(y, "ssm_scan: y");
     if (H < 1 || G < 1 || H % G != 0 || P < 1 || N < 1) fail("ssm_scan: %d heads, %d groups, %d x %d states are not supported", H, G, N, P);
-    if (N > 1024) fail("ssm_scan: a state of %d rows is not supported (up to 1024)", N);
     if (xbc.cols != static_cast<int64_t>(H) * P + 2 * G * N) fail("ssm_scan: x, B, C rows must be %d wide", H * P + 2 * G * N);
     if (dt_col < 0 || dt_col + H > proj.cols || proj.rows != xbc.rows) fail("ssm_scan: the step sizes lie outside their rows");
     if (y.rows != xbc.rows || y.cols != static_cast<int64_t>(H) * P) fail("ssm_scan: y must be [%lld, %d]", (long long)xbc.rows, H * P);
@@ -112,8 +113,11 @@ void ssm_scan(const Tensor2& xbc, const Tensor2& proj, int dt_col, const float* 
         fail("ssm_scan: the workspace holds %zu floats, %zu are needed", workspace_floats, ssm_scan_workspace_floats(T, st.n_seqs, H, P, N));
     check(mllm_ssm_scan(static_cast<const float*>(xbc.data), i32(xbc.stride), static_cast<const float*>(proj.data) + dt_col, i32(proj.stride),
                         dt_bias, A_log, skip, st.cu_q, st.state_slots, st.state, st.slot_floats, scan_offset, static_cast<float*>(y.data),
-                        i32(y.stride), T, st.n_seqs, max_q, H, P, N, G, st.write ? 1 : 0, workspace, stream), "ssm_scan");
+                        i32(y.stride), static_cast<size_t>(y.rows) * y.stride, T, st.n_seqs, max_q, H, P, N, G, st.write ? 1 : 0, workspace,
+                        stream), "ssm_scan");
 }
+
+int ssm_scan_parts(int N) { return mllm_ssm_scan_parts(N); }
 
 size_t ssm_scan_workspace_floats(int tokens, int n_seqs, int H, int P, int N) {
     return mllm_ssm_scan_workspace_floats(tokens, n_seqs, H, P, N);
@@ -162,8 +166,8 @@ void latent_absorb(const Tensor2& q, const Tensor2& w_uk, const Tensor2& qa, con
     need_act(q, "latent_absorb: q");
     const int E = sh.kv_rank + sh.rot_dim;
     if (q.cols != static_cast<int64_t>(sh.n_heads) * (sh.plain_dim + sh.rot_dim)) fail("latent_absorb: q must be [T, %d]", sh.n_heads * (sh.plain_dim + sh.rot_dim));
-    if (w_uk.dtype != q.dtype || w_uk.rows != static_cast<int64_t>(sh.n_heads) * sh.plain_dim || w_uk.cols != sh.kv_rank)
-        fail("latent_absorb: the key expansion must be [%d, %d] %s", sh.n_heads * sh.plain_dim, sh.kv_rank, dtype_name(q.dtype));
+    if (w_uk.dtype != q.dtype || w_uk.cols != static_cast<int64_t>(sh.n_heads) * sh.plain_dim || w_uk.rows != sh.kv_rank)
+        fail("latent_absorb: the transposed key expansion must be [%d, %d] %s", sh.kv_rank, sh.n_heads * sh.plain_dim, dtype_name(q.dtype));
     if (qa.dtype != q.dtype || qa.rows != q.rows || qa.cols != static_cast<int64_t>(sh.n_heads) * E) fail("latent_absorb: qa must be [T, %d]", sh.n_heads * E);
     if (positions == nullptr) fail("latent_absorb: positions are needed");
     check(mllm_latent_absorb(q.data, i32(q.stride), w_uk.data, i32(w_uk.stride), qa.data, i32(qa.stride), positions, i32(q.rows), sh.n_heads,
@@ -190,19 +194,21 @@ void latent_attention(const Tensor2& qa, const LatentPages& pages, const LatentS
     // the matrix-core kernel: one workgroup per 64 (token, head) rows of a sequence
     if (tuning().latent_tiles && qa.dtype == BF16 && pages.latent_t.data != nullptr && step.cu_q != nullptr &&
         step.ctx_len != nullptr && step.n_seqs > 0 && qa.contiguous() && o_lat.contiguous()) {
-        const long long rows = static_cast<long long>(T) * sh.n_heads, tiles = rows / 64 + step.n_seqs;
+        const bool single = step.max_q_len == 1 && T == step.n_seqs;        // one token a sequence: tiles are numbered directly
+        const long long rows = static_cast<long long>(T) * sh.n_heads,
+                        tiles = single ? static_cast<long long>(step.n_seqs) * ((sh.n_heads + 63) / 64) : rows / 64 + step.n_seqs;
         if (tiles < (1ll << 31)) {
-            // Few workgroups (decoding): every row's key tiles are spread over several, so that about 512
+            // Few workgroups (decoding): every row's key tiles are spread over several, so that about 256
             // workgroups stream the pages instead of one per sequence walking its tiles one after the other.
             const int keys = window > 0 ? std::min(window, std::max(step.max_ctx_len, 1)) : std::max(step.max_ctx_len, 1);
             int nsplit = 1;
             if (workspace != nullptr && tiles < 256) {
-                nsplit = static_cast<int>(std::min<long long>({(keys + 63) / 64 + 1, 512 / tiles, LATENT_SPLIT_ROWS / std::max<long long>(rows, 1)}));
+                nsplit = static_cast<int>(std::min<long long>({(keys + 63) / 64 + 1, 256 / tiles, 64, LATENT_SPLIT_ROWS / std::max<long long>(rows, 1)}));
                 if (nsplit < 2 || static_cast<size_t>(rows) * nsplit * (sh.kv_rank + 2) > workspace_floats) nsplit = 1;
             }
             const int rc = mllm_latent_attention_tiles(qa.data, pages.rows.data, pages.latent_t.data, step.block_tables, step.max_blocks, step.cu_q,
                                                        step.ctx_len, step.n_seqs, static_cast<int>(tiles), sh.n_heads, sh.kv_rank, sh.rot_dim,
-                                                       pages.page_size, scale, window, o_lat.data, static_cast<int>(rows), nsplit, workspace, stream);
+                                                       pages.page_size, scale, window, o_lat.data, static_cast<int>(rows), nsplit, workspace, single ? 1 : 0, stream);
             if (rc == 0) { tuning().seen.latent_tile_launches += 1; return; }
             if (rc != -2) check(rc, "latent_attention (tiles)");
         }

@@ -66,10 +66,12 @@ latent_prepare_kernel(const float* __restrict__ dq, int ld_dq, int Rq, const flo
     for (int i = rot_dims + lane; i < Dr; i += 64) o[R + i] = from_float<T>(row[R + i]);
 }
 
-// Queries into the latent space. q rows: per head [Dn plain | Dr to be turned]; w_uk [H * Dn, R] (row h*Dn + d
-// expands latent column r into the head's plain key dimension d). For 8 tokens and one head a workgroup:
-//   qa[t, h, r] = sum_d q[t, h, d] * w_uk[h*Dn + d, r]      (thread per r: the weight reads are coalesced)
+// Queries into the latent space. q rows: per head [Dn plain | Dr to be turned]; w_ukt [R, H * Dn] is the key
+// expansion transposed (column h*Dn + d of row r expands latent column r into the head's plain key dimension d).
+// For 8 tokens and one head a workgroup:
+//   qa[t, h, r] = sum_d q[t, h, d] * w_ukt[r, h*Dn + d]      (thread per r)
 //   qa[t, h, R + i] = the turned rotary part of q[t, h]
+// (Any dtype and sizes; bfloat16 at sizes in steps of 32 goes to head_linear_mfma_kernel.)
 template <typename T>
 __global__ void __launch_bounds__(256)
 latent_absorb_kernel(const T* __restrict__ q, int ldq, const T* __restrict__ w_uk, int ldw, T* __restrict__ qa, int ldqa,
@@ -85,9 +87,9 @@ latent_absorb_kernel(const T* __restrict__ q, int ldq, const T* __restrict__ w_u
     __syncthreads();
     for (int r = blockIdx.x * 256 + threadIdx.x; r < R; r += gridDim.x * 256) {
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        const T* wcol = w_uk + static_cast<size_t>(h) * Dn * ldw + r;
+        const T* wrow = w_uk + static_cast<size_t>(r) * ldw + static_cast<size_t>(h) * Dn;
         for (int d = 0; d < Dn; ++d) {
-            const float wv = to_float(wcol[static_cast<size_t>(d) * ldw]);
+            const float wv = to_float(wrow[d]);
 #pragma unroll
             for (int tt = 0; tt < 8; ++tt) acc[tt] += q_s[tt * Dn + d] * wv;
         }
@@ -110,6 +112,77 @@ latent_absorb_kernel(const T* __restrict__ q, int ldq, const T* __restrict__ w_u
                 }
             } else {
                 const int c = k - Dr / 2;
+                if (c >= rot_dims) dst[c] = src[c];
+            }
+        }
+    }
+}
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+union Frag8 {
+    bf16x8 v;
+    u32x4 q;
+    uint32_t w[4];
+};
+
+// One small product per head on the matrix cores (bfloat16, fp32 sums), operands straight from memory:
+//   out[t, h*out_hs + n] = sum_k a[t, h*a_hs + k] * w[(h*w_head_rows + n) * ldw + h*w_head_cols + k],  n < N, k < K
+// (w_head_rows = N, w_head_cols = 0: every head has its own rows of w; w_head_rows = 0, w_head_cols = K: its own
+// columns). A workgroup takes 64 tokens, one head and 64 values of n; a wavefront 16 tokens: the weights are the
+// MFMA's A operand, so a lane ends up with four neighbouring n of one token. K is a multiple of 32; rows and head
+// offsets are 16-byte aligned. With `positions`, the workgroups of the first n tile also carry the `tail` columns
+// behind a head's K inputs over to behind its N outputs, the first rot_dims of them turned in interleaved pairs.
+__global__ void __launch_bounds__(256)
+head_linear_mfma_kernel(const bf16_t* __restrict__ a, int lda, int a_hs, const bf16_t* __restrict__ w, int ldw, int w_head_rows,
+                        int w_head_cols, bf16_t* __restrict__ out, int ldo, int out_hs, int n_tokens, int N, int K,
+                        const int* __restrict__ positions, int tail, int rot_dims, double log2_base) {
+    const int lane = threadIdx.x % 64, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int G = lane / 16, c16 = lane % 16;
+    const int h = blockIdx.y, t0 = blockIdx.x * 64, n_base = blockIdx.z * 64;
+    const int tok = min(t0 + 16 * wave + c16, n_tokens - 1);
+    const bf16_t* arow = a + static_cast<size_t>(tok) * lda + static_cast<size_t>(h) * a_hs + 8 * G;
+    const bf16_t* wbase = w + static_cast<size_t>(h) * w_head_rows * ldw + static_cast<size_t>(h) * w_head_cols + 8 * G;
+    const bf16_t* wrow[4];
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) wrow[ct] = wbase + static_cast<size_t>(min(n_base + 16 * ct + c16, N - 1)) * ldw;
+    f32x4 acc[4];
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) acc[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < K; k += 32) {
+        Frag8 af, wf[4];
+        af.q = *reinterpret_cast<const u32x4*>(arow + k);
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) wf[ct].q = *reinterpret_cast<const u32x4*>(wrow[ct] + k);
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[ct].v, af.v, acc[ct], 0, 0, 0);
+    }
+    if (t0 + 16 * wave + c16 < n_tokens) {
+        bf16_t* orow = out + static_cast<size_t>(tok) * ldo + static_cast<size_t>(h) * out_hs;
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+            const int n = n_base + 16 * ct + 4 * G;            // acc[ct][r] is output n + r of this lane's token
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n + r < N) orow[n + r] = float_to_bf16(acc[ct][r]);
+        }
+    }
+    if (positions != nullptr && blockIdx.z == 0) {
+        const int nt = min(64, n_tokens - t0), per = tail / 2 + tail;
+        for (int i = threadIdx.x; i < nt * per; i += 256) {
+            const int tt = i / per, k = i % per;
+            const bf16_t* src = a + static_cast<size_t>(t0 + tt) * lda + static_cast<size_t>(h) * a_hs + K;
+            bf16_t* dst = out + static_cast<size_t>(t0 + tt) * ldo + static_cast<size_t>(h) * out_hs + N;
+            if (k < tail / 2) {
+                if (k < rot_dims / 2) {
+                    float u, v;
+                    turn_pair(to_float(src[2 * k]), to_float(src[2 * k + 1]), positions[t0 + tt], k, log2_base, rot_dims, u, v);
+                    dst[2 * k] = float_to_bf16(u);
+                    dst[2 * k + 1] = float_to_bf16(v);
+                }
+            } else {
+                const int c = k - tail / 2;
                 if (c >= rot_dims) dst[c] = src[c];
             }
         }
@@ -228,15 +301,6 @@ latent_expand_kernel(const T* __restrict__ o_lat, int ldo, const T* __restrict__
     }
 }
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-union Frag8 {
-    bf16x8 v;
-    u32x4 q;
-    uint32_t w[4];
-};
-
 // Prompt portions on the matrix cores (bfloat16, fp32 softmax). A query row is a (token, head) pair; a
 // sequence's rows are numbered token by token, head by head, and a workgroup takes 64 consecutive rows (its
 // four wavefronts 16 each), which lie on few neighbouring tokens, so they share their keys: one staging of a
@@ -252,7 +316,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))
 latent_prefill_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
                       const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
                       const int* __restrict__ ctx_len, int n_seqs, int H, int page_size, float scale_log2e, int window,
-                      bf16_t* __restrict__ o_lat, int nsplit, float* __restrict__ partials) {
+                      bf16_t* __restrict__ o_lat, int nsplit, float* __restrict__ partials, int single_tokens) {
     constexpr int E = 32 * KS, R = 16 * DT, BN = 64, KSTRIDE = E + 8, VSTRIDE = BN + 8, CH = E / 8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     bf16_t* Ks = reinterpret_cast<bf16_t*>(smem);                    // [BN][KSTRIDE]
@@ -260,12 +324,21 @@ latent_prefill_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ 
     int* sm_table = reinterpret_cast<int*>(Vt + R * VSTRIDE);        // the sequence's block table
 
     int tile = gridDim.x - 1 - blockIdx.x, b = 0, q_begin = 0, q_len = 0;
-    for (; b < n_seqs; ++b) {
-        q_begin = cu_q[b];
-        q_len = cu_q[b + 1] - q_begin;
-        const int nt = (q_len * H + 63) / 64;
-        if (tile < nt) break;
-        tile -= nt;
+    if (single_tokens) {
+        // every sequence brings one token: its tiles follow from the tile's index, without the walk over the
+        // sequences below, whose every step waits for a load
+        const int per = (H + 63) / 64;
+        b = tile / per;
+        tile -= b * per;
+        if (b < n_seqs) { q_begin = b; q_len = 1; }
+    } else {
+        for (; b < n_seqs; ++b) {
+            q_begin = cu_q[b];
+            q_len = cu_q[b + 1] - q_begin;
+            const int nt = (q_len * H + 63) / 64;
+            if (tile < nt) break;
+            tile -= nt;
+        }
     }
     if (b >= n_seqs) return;                       // surplus workgroup; the whole workgroup leaves
     const int tid = threadIdx.x, lane = tid % 64;
@@ -413,25 +486,36 @@ latent_prefill_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ 
     }
 }
 
-// The splits' states of a row merged: o = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s. One wavefront per row.
+// The splits' states of a row merged: o = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s. One wavefront per row
+// (up to 64 splits: lane s weighs split s; the weights pass through LDS; the outputs are added in the order of
+// the splits, four columns a lane at a time, every load issued before the first use).
 __global__ void __launch_bounds__(256)
 latent_merge_kernel(const float* __restrict__ partials, int n_rows, int nsplit, int R, bf16_t* __restrict__ o_lat) {
+    __shared__ float weights[4][64];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
     const int row = blockIdx.x * 4 + wave;
     if (row >= n_rows) return;
     const float* st = partials + static_cast<size_t>(row) * nsplit * (R + 2);
-    float M = -INFINITY;
-    for (int sp = 0; sp < nsplit; ++sp) M = fmaxf(M, st[static_cast<size_t>(sp) * (R + 2)]);
-    float L = 0.f;
-    for (int sp = 0; sp < nsplit; ++sp) L += fast_exp2(st[static_cast<size_t>(sp) * (R + 2)] - M) * st[static_cast<size_t>(sp) * (R + 2) + 1];
-    const float inv = 1.0f / L;
-    for (int c = lane; c < R; c += 64) {
-        float acc = 0.f;
+    const float* mine = st + static_cast<size_t>(min(lane, nsplit - 1)) * (R + 2);
+    const float m = lane < nsplit ? mine[0] : -INFINITY, l = lane < nsplit ? mine[1] : 0.f;
+    const float M = wave_max(m);
+    const float wgt = fast_exp2(m - M);
+    const float inv = 1.0f / wave_sum(wgt * l);
+    weights[wave][lane] = wgt * inv;
+    wave_lds_sync();
+    for (int c = 4 * lane; c < R; c += 256) {
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
         for (int sp = 0; sp < nsplit; ++sp) {
-            const float* one = st + static_cast<size_t>(sp) * (R + 2);
-            acc += fast_exp2(one[0] - M) * one[2 + c];
+            // (R + 2 is even and c a multiple of 4: the columns of a state are 8-byte aligned)
+            const float2 a = *reinterpret_cast<const float2*>(st + static_cast<size_t>(sp) * (R + 2) + 2 + c);
+            const float2 b = *reinterpret_cast<const float2*>(st + static_cast<size_t>(sp) * (R + 2) + 4 + c);
+            const float ws = weights[wave][sp];
+            acc.x += ws * a.x; acc.y += ws * a.y; acc.z += ws * b.x; acc.w += ws * b.y;
         }
-        o_lat[static_cast<size_t>(row) * R + c] = float_to_bf16(acc * inv);
+        uint2 pk;
+        pk.x = pack_bf16x2(acc.x, acc.y);
+        pk.y = pack_bf16x2(acc.z, acc.w);
+        *reinterpret_cast<uint2*>(o_lat + static_cast<size_t>(row) * R + c) = pk;
     }
 }
 
@@ -461,15 +545,24 @@ int mllm_latent_prepare(const float* dq, int ld_dq, int Rq, const float* wq, voi
     return 0;
 }
 
-// See latent_absorb_kernel. -1: rot_dims odd or beyond Dr, Dr odd; -2: Dn too large for the LDS.
+// See latent_absorb_kernel; w_uk is the key expansion transposed, [R, H * Dn]. -1: rot_dims odd or beyond Dr, Dr
+// odd; -2: Dn too large for the LDS.
 int mllm_latent_absorb(const void* q, int ldq, const void* w_uk, int ldw, void* qa, int ldqa, const int* positions, int T, int H,
                        int Dn, int Dr, int R, double base, int rot_dims, int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
     if (rot_dims < 0 || rot_dims % 2 != 0 || rot_dims > Dr || Dr % 2 != 0 || !(base > 0)) return -1;
+    const double l2 = log2(base);
+    const auto aligned16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+    if (dtype == MLLM_BF16 && Dn % 32 == 0 && ldq % 8 == 0 && (Dn + Dr) % 8 == 0 && ldw % 8 == 0 && aligned16(q) && aligned16(w_uk)) {
+        head_linear_mfma_kernel<<<dim3((T + 63) / 64, H, (R + 63) / 64), 256, 0, stream>>>(
+            static_cast<const bf16_t*>(q), ldq, Dn + Dr, static_cast<const bf16_t*>(w_uk), ldw, 0, Dn, static_cast<bf16_t*>(qa), ldqa, R + Dr,
+            T, R, Dn, positions, Dr, rot_dims, l2);
+        MLLM_LAUNCH_CHECK();
+        return 0;
+    }
     const size_t lds = static_cast<size_t>(8) * Dn * sizeof(float);
     if (lds > 64 * 1024) return -2;
     const dim3 grid((R + 255) / 256, H, (T + 7) / 8);
-    const double l2 = log2(base);
     if (dtype == MLLM_F32)
         latent_absorb_kernel<float><<<grid, 256, lds, stream>>>(static_cast<const float*>(q), ldq, static_cast<const float*>(w_uk), ldw,
                                                                 static_cast<float*>(qa), ldqa, positions, T, H, Dn, Dr, R, l2, rot_dims);
@@ -522,17 +615,18 @@ int mllm_latent_attention(const void* qa, int ldqa, const void* pages, const int
 
 // The matrix-core kernel (see latent_prefill_kernel): qa [T*H, E] and o_lat [T*H, R] contiguous bfloat16.
 // nsplit > 1: every row's key tiles are shared by nsplit workgroups whose states meet in `partials`
-// (n_rows * nsplit * (R + 2) floats, n_rows = T*H) and are merged by a second kernel. n_tiles_upper: an upper bound of sum over sequences of ceil(q_len * H / 64). Returns -2 when the
+// (n_rows * nsplit * (R + 2) floats, n_rows = T*H) and are merged by a second kernel. single_tokens != 0: every
+// sequence brings exactly one token (n_tiles_upper is then n_seqs * ceil(H / 64)). n_tiles_upper: an upper bound of sum over sequences of ceil(q_len * H / 64). Returns -2 when the
 // sizes are not ones it is built for (E and R among (128, 96), (96, 64), (160, 128), (288, 256), (576, 512);
 // page sizes 8 to 64, powers of two; a block table that fits the LDS beside the tiles): the caller then runs
 // mllm_latent_attention.
 int mllm_latent_attention_tiles(const void* qa, const void* k_pages, const void* vt_pages, const int* block_tables,
                                 int max_blocks, const int* cu_q, const int* ctx_len, int n_seqs, int n_tiles_upper, int H,
                                 int R, int Dr, int page_size, float scale, int window, void* o_lat, int n_rows, int nsplit,
-                                float* partials, hipStream_t stream) {
+                                float* partials, int single_tokens, hipStream_t stream) {
     if (n_seqs <= 0 || n_tiles_upper <= 0) return 0;
     const int E = R + Dr;
-    if (nsplit < 1 || nsplit > 65535 || (nsplit > 1 && (partials == nullptr || n_rows < 1))) return -1;
+    if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (partials == nullptr || n_rows < 1))) return -1;
     if (E % 32 != 0 || R % 16 != 0 || page_size < 8 || page_size > 64 || (page_size & (page_size - 1)) != 0) return -2;
     if (((reinterpret_cast<uintptr_t>(qa) | reinterpret_cast<uintptr_t>(k_pages) | reinterpret_cast<uintptr_t>(vt_pages) |
           reinterpret_cast<uintptr_t>(o_lat)) & 15) != 0)
@@ -552,7 +646,7 @@ int mllm_latent_attention_tiles(const void* qa, const void* k_pages, const void*
         latent_prefill_kernel<KS, DT><<<dim3(n_tiles_upper, nsplit), 256, lds, stream>>>(                            \
             static_cast<const bf16_t*>(qa), static_cast<const bf16_t*>(k_pages), static_cast<const bf16_t*>(vt_pages), \
             block_tables, max_blocks, cu_q, ctx_len, n_seqs, H, page_size, sl2, window, static_cast<bf16_t*>(o_lat), \
-            nsplit, partials);                                                                                       \
+            nsplit, partials, single_tokens);                                                                        \
         MLLM_LAUNCH_CHECK();                                                                                         \
         if (nsplit > 1) {                                                                                            \
             latent_merge_kernel<<<(n_rows + 3) / 4, 256, 0, stream>>>(partials, n_rows, nsplit, R,                   \
@@ -569,6 +663,14 @@ int mllm_latent_attention_tiles(const void* qa, const void* k_pages, const void*
 int mllm_latent_expand(const void* o_lat, int ldo, const void* w_uv, int ldw, void* out, int ldout, int T, int H, int Dv, int R,
                        int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
+    if (dtype == MLLM_BF16 && R % 32 == 0 && ldo % 8 == 0 && ldw % 8 == 0 && (reinterpret_cast<uintptr_t>(o_lat) & 15) == 0 &&
+        (reinterpret_cast<uintptr_t>(w_uv) & 15) == 0) {
+        head_linear_mfma_kernel<<<dim3((T + 63) / 64, H, (Dv + 63) / 64), 256, 0, stream>>>(
+            static_cast<const bf16_t*>(o_lat), ldo, R, static_cast<const bf16_t*>(w_uv), ldw, Dv, 0, static_cast<bf16_t*>(out), ldout, Dv, T, Dv,
+            R, nullptr, 0, 0, 0.0);
+        MLLM_LAUNCH_CHECK();
+        return 0;
+    }
     const dim3 grid((H * Dv + 3) / 4, std::min((T + 7) / 8, 64));
     if (dtype == MLLM_F32)
         latent_expand_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(o_lat), ldo, static_cast<const float*>(w_uv), ldw,

@@ -15,13 +15,18 @@ template <typename OutT, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES)
 rmsnorm_kernel(const float* __restrict__ x, int ldx, const int* __restrict__ rows, const float* __restrict__ w,
                const float* __restrict__ gate, int ldg, OutT* __restrict__ y, int ldy, int n, int D, int groups,
-               float eps) {
+               float eps, int parts, size_t part_stride) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
     const long long pair = static_cast<long long>(blockIdx.x) * WAVES + wave;
     if (pair >= static_cast<long long>(n) * groups) return;
     const int r = static_cast<int>(pair / groups), g = static_cast<int>(pair % groups), Dg = D / groups;
     const int src = rows ? rows[r] : r;
     const float* xr = x + static_cast<size_t>(src) * ldx + g * Dg;
+    auto input = [&](int i) {
+        float a = xr[i];
+        for (int part = 1; part < parts; ++part) a += xr[part * part_stride + i];
+        return a;
+    };
     const float* gr = gate ? gate + static_cast<size_t>(src) * ldg + g * Dg : nullptr;
     const float* wr = w + g * Dg;
     OutT* yr = y + static_cast<size_t>(r) * ldy + g * Dg;
@@ -33,14 +38,14 @@ rmsnorm_kernel(const float* __restrict__ x, int ldx, const int* __restrict__ row
         const int i = lane + 64 * u;
         float a = 0.f;
         if (i < Dg) {
-            a = xr[i];
+            a = input(i);
             if (gr) { const float z = gr[i]; a *= z * sigmoid_precise(z); }
         }
         v[u] = a;
         ss += a * a;
     }
     for (int i = lane + 512; i < Dg; i += 64) {
-        float a = xr[i];
+        float a = input(i);
         if (gr) { const float z = gr[i]; a *= z * sigmoid_precise(z); }
         ss += a * a;
     }
@@ -51,7 +56,7 @@ rmsnorm_kernel(const float* __restrict__ x, int ldx, const int* __restrict__ row
         if (i < Dg) yr[i] = from_float<OutT>(v[u] * inv * wr[i]);
     }
     for (int i = lane + 512; i < Dg; i += 64) {
-        float a = xr[i];
+        float a = input(i);
         if (gr) { const float z = gr[i]; a *= z * sigmoid_precise(z); }
         yr[i] = from_float<OutT>(a * inv * wr[i]);
     }
@@ -94,6 +99,115 @@ rmsnorm_add_kernel(float* __restrict__ y, const float* __restrict__ w, const flo
     }
 }
 
+// The same two norms for rows whose parts are multiples of 4 and at most 2,048 long, 16-byte aligned: the part
+// lives in registers as float4, and every load is issued without a condition, from a clamped index, before the
+// first use (a load under a condition waits for all loads in flight, and a row of 768 then costs eight round trips).
+// `parts` > 1: the input is the sum of that many arrays `part_stride` floats apart (partial results of a kernel
+// that splits a sum over workgroups), added in the order of their index.
+template <typename OutT, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
+rmsnorm_vec_kernel(const float* __restrict__ x, int ldx, const int* __restrict__ rows, const float* __restrict__ w,
+                   const float* __restrict__ gate, int ldg, OutT* __restrict__ y, int ldy, int n, int D, int groups,
+                   float eps, int parts, size_t part_stride) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
+    const long long pair = static_cast<long long>(blockIdx.x) * WAVES + wave;
+    if (pair >= static_cast<long long>(n) * groups) return;
+    const int r = static_cast<int>(pair / groups), g = static_cast<int>(pair % groups), Dg = D / groups;
+    const int src = rows ? rows[r] : r;
+    const float4* xr = reinterpret_cast<const float4*>(x + static_cast<size_t>(src) * ldx + g * Dg);
+    const float4* gr = reinterpret_cast<const float4*>(gate ? gate + static_cast<size_t>(src) * ldg + g * Dg : x);
+    const float4* wr = reinterpret_cast<const float4*>(w + g * Dg);
+    const int nq = Dg / 4, n_u = (nq + 63) / 64;
+    float4 v[8], gg[8], ww[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        if (u < n_u) v[u] = xr[min(lane + 64 * u, nq - 1)];
+    for (int part = 1; part < parts; ++part) {
+        const float4* xp = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(xr) + part * part_stride);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (u < n_u) {
+                const float4 a = xp[min(lane + 64 * u, nq - 1)];
+                v[u].x += a.x; v[u].y += a.y; v[u].z += a.z; v[u].w += a.w;
+            }
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        if (u < n_u) {
+            const int i = min(lane + 64 * u, nq - 1);
+            gg[u] = gr[i];
+            ww[u] = wr[i];
+        }
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        if (u < n_u) {
+            if (gate) {
+                v[u].x *= gg[u].x * sigmoid_precise(gg[u].x); v[u].y *= gg[u].y * sigmoid_precise(gg[u].y);
+                v[u].z *= gg[u].z * sigmoid_precise(gg[u].z); v[u].w *= gg[u].w * sigmoid_precise(gg[u].w);
+            }
+            if (lane + 64 * u < nq) ss += (v[u].x * v[u].x + v[u].y * v[u].y) + (v[u].z * v[u].z + v[u].w * v[u].w);
+        }
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(Dg) + eps);
+    OutT* yr = y + static_cast<size_t>(r) * ldy + g * Dg;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int i = lane + 64 * u;
+        if (u < n_u && i < nq) {
+            const float o0 = v[u].x * inv * ww[u].x, o1 = v[u].y * inv * ww[u].y, o2 = v[u].z * inv * ww[u].z, o3 = v[u].w * inv * ww[u].w;
+            if (sizeof(OutT) == 2) {
+                uint2 pk;
+                pk.x = pack_bf16x2(o0, o1);
+                pk.y = pack_bf16x2(o2, o3);
+                *reinterpret_cast<uint2*>(yr + 4 * i) = pk;
+            } else {
+                *reinterpret_cast<float4*>(yr + 4 * i) = make_float4(o0, o1, o2, o3);
+            }
+        }
+    }
+}
+
+template <int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
+rmsnorm_add_vec_kernel(float* __restrict__ y, const float* __restrict__ w, const float* __restrict__ scale, float mult,
+                       float eps, float* __restrict__ x, int n, int D, int clear) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
+    const int r = blockIdx.x * WAVES + wave;
+    if (r >= n) return;
+    float4* yr = reinterpret_cast<float4*>(y + static_cast<size_t>(r) * D);
+    float4* xr = reinterpret_cast<float4*>(x + static_cast<size_t>(r) * D);
+    const float4* wr = reinterpret_cast<const float4*>(w);
+    const float4* sr = reinterpret_cast<const float4*>(scale ? scale : w);
+    const int nq = D / 4, n_u = (nq + 63) / 64;
+    float4 v[8], xx[8], ww[8], sc[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        if (u < n_u) v[u] = yr[min(lane + 64 * u, nq - 1)];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        if (u < n_u) {
+            const int i = min(lane + 64 * u, nq - 1);
+            xx[u] = xr[i];
+            ww[u] = wr[i];
+            sc[u] = sr[i];
+        }
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        if (u < n_u && lane + 64 * u < nq) ss += (v[u].x * v[u].x + v[u].y * v[u].y) + (v[u].z * v[u].z + v[u].w * v[u].w);
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(D) + eps);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int i = lane + 64 * u;
+        if (u < n_u && i < nq) {
+            const float4 s4 = scale ? make_float4(sc[u].x * mult, sc[u].y * mult, sc[u].z * mult, sc[u].w * mult) : make_float4(mult, mult, mult, mult);
+            xr[i] = make_float4(xx[u].x + s4.x * (v[u].x * inv * ww[u].x), xx[u].y + s4.y * (v[u].y * inv * ww[u].y),
+                                xx[u].z + s4.z * (v[u].z * inv * ww[u].z), xx[u].w + s4.w * (v[u].w * inv * ww[u].w));
+            if (clear) yr[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+}
+
 // out[t, i] = g sigmoid(alpha g) (u + 1) with g = min(gate[t, i], limit), u = clamp(up[t, i], -limit, limit).
 template <typename T>
 __global__ void glu_clamped_kernel(const T* gate, int ldg, const T* up, int ldu, T* out, int ldo,     // (out may be gate)
@@ -118,17 +232,29 @@ __global__ void fill_zero_kernel(float4* __restrict__ p, size_t n4) {
 extern "C" {
 
 // y = rmsnorm(x[rows]) in `groups` equal parts of the D columns, optionally gated (see the kernel).
-// x and gate fp32 with row strides ldx / ldg; y in out_dtype with row stride ldy. -1: D is no multiple of groups.
+// x and gate fp32 with row strides ldx / ldg; y in out_dtype with row stride ldy. With parts > 1, x is the sum of
+// `parts` arrays part_stride floats apart. -1: D is no multiple of groups.
 int mllm_rmsnorm(const float* x, int ldx, const int* rows, const float* w, const float* gate, int ldg, void* y, int ldy,
-                 int n, int D, int groups, float eps, int out_dtype, hipStream_t stream) {
+                 int n, int D, int groups, float eps, int out_dtype, int parts, size_t part_stride, hipStream_t stream) {
     if (n <= 0 || D <= 0) return 0;
-    if (groups < 1 || D % groups != 0) return -1;
+    if (groups < 1 || D % groups != 0 || parts < 1) return -1;
     const long long pairs = static_cast<long long>(n) * groups;
-    const int blocks = static_cast<int>((pairs + 3) / 4);
-    if (out_dtype == MLLM_F32)
-        rmsnorm_kernel<float, 4><<<blocks, 256, 0, stream>>>(x, ldx, rows, w, gate, ldg, static_cast<float*>(y), ldy, n, D, groups, eps);
-    else
-        rmsnorm_kernel<bf16_t, 4><<<blocks, 256, 0, stream>>>(x, ldx, rows, w, gate, ldg, static_cast<bf16_t*>(y), ldy, n, D, groups, eps);
+    const int Dg = D / groups, esz = out_dtype == MLLM_F32 ? 4 : 2;
+    const bool vec = Dg % 4 == 0 && Dg <= 2048 && ldx % 4 == 0 && (gate == nullptr || ldg % 4 == 0) && part_stride % 4 == 0 &&
+                     (static_cast<size_t>(ldy) * esz) % 16 == 0 && (static_cast<size_t>(Dg) * esz) % 8 == 0 &&
+                     ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(gate) |
+                       reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    // (workgroups start at a limited rate: many rows go eight to a workgroup)
+#define RMS(KERNEL, TYPE, WAVES)                                                                                        \
+    KERNEL<TYPE, WAVES><<<static_cast<int>((pairs + WAVES - 1) / WAVES), 64 * WAVES, 0, stream>>>(                      \
+        x, ldx, rows, w, gate, ldg, static_cast<TYPE*>(y), ldy, n, D, groups, eps, parts, part_stride)
+    if (vec) {
+        if (out_dtype == MLLM_F32) { if (pairs >= 512) RMS(rmsnorm_vec_kernel, float, 8); else RMS(rmsnorm_vec_kernel, float, 4); }
+        else { if (pairs >= 512) RMS(rmsnorm_vec_kernel, bf16_t, 8); else RMS(rmsnorm_vec_kernel, bf16_t, 4); }
+    } else {
+        if (out_dtype == MLLM_F32) RMS(rmsnorm_kernel, float, 4); else RMS(rmsnorm_kernel, bf16_t, 4);
+    }
+#undef RMS
     MLLM_LAUNCH_CHECK();
     return 0;
 }
@@ -136,7 +262,12 @@ int mllm_rmsnorm(const float* x, int ldx, const int* rows, const float* w, const
 int mllm_rmsnorm_add(float* y, const float* w, const float* scale, float mult, float eps, float* x, int n, int D,
                      int clear, hipStream_t stream) {
     if (n <= 0 || D <= 0) return 0;
-    rmsnorm_add_kernel<4><<<(n + 3) / 4, 256, 0, stream>>>(y, w, scale, mult, eps, x, n, D, clear);
+    const bool vec = D % 4 == 0 && D <= 2048 &&
+                     ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(scale) |
+                       reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    if (vec && n >= 512) rmsnorm_add_vec_kernel<8><<<(n + 7) / 8, 512, 0, stream>>>(y, w, scale, mult, eps, x, n, D, clear);
+    else if (vec) rmsnorm_add_vec_kernel<4><<<(n + 3) / 4, 256, 0, stream>>>(y, w, scale, mult, eps, x, n, D, clear);
+    else rmsnorm_add_kernel<4><<<(n + 3) / 4, 256, 0, stream>>>(y, w, scale, mult, eps, x, n, D, clear);
     MLLM_LAUNCH_CHECK();
     return 0;
 }

@@ -3,7 +3,7 @@
 // in a per-request slot. Everything here is fp32.
 //
 // A request's slot holds [taps - 1][channels] convolution inputs (oldest first), then the scan's state
-// laid out [head][p][n] (n contiguous).
+// laid out [head][n][p] (p contiguous).
 #include <algorithm>
 
 #include "common.h"
@@ -67,21 +67,25 @@ __global__ void conv_carry_kernel(const float* __restrict__ proj, int ld, int co
 // The scan. For head h (group g = h / (H / G)) and token t, in order:
 //   dt = softplus(raw_dt[t, h] + dt_bias[h]);  a = exp(-exp(A_log[h]) dt)
 //   S[n, p] = a S[n, p] + dt B[t, g, n] x[t, h, p];   y[t, h, p] = sum_n S[n, p] C[t, g, n] + D[h] x[t, h, p]
-// One wavefront per (chunk of a sequence's portion, head, 64 / LANES_N values of p): LANES_N consecutive
-// lanes share a p and split n (lane l of the group holds n = l, l + LANES_N, ...: up to NPT of them in
-// registers), so the sum over n is a sum inside the lane group and no wavefront waits for another. The next
-// token's operands are requested before this token's are used. xbc rows: [x: H*P | B: G*N | C: G*N].
+// One wavefront per (chunk of a sequence's portion, head, 64 values of p, slice of NS values of n): a lane owns
+// one p and keeps its NS state values in registers, so B and C of the slice are the same for the whole wavefront
+// (they arrive as scalars) and x is one coalesced load. The sum over n is split over the slices: slice s leaves its
+// share in y + s * part_stride, and the reader (the gated norm) adds the shares in the order of s. The state in a
+// slot is laid out [head][n][p] (p contiguous). xbc rows: [x: H*P | B: G*N | C: G*N].
 //
 // A portion longer than `chunk` tokens is cut into chunks that are scanned side by side: the first starts
 // from the slot's state, the others from zero, and each leaves its last state in `chunk_state`
-// ([chunk][H][P][N]) and, per token, the logarithm of the decay accumulated since its chunk began in `cumlog`
+// ([chunk][H][N][P]) and, per token, the logarithm of the decay accumulated since its chunk began in `cumlog`
 // ([T, H]). ssm_chunk_join_kernel then adds what the earlier chunks contribute. A portion of one chunk
 // (decoding) is finished here and its state goes straight back to the slot.
 struct ChunkOf {
     int b, k, n_chunks, first_chunk;      // sequence, chunk within it, chunks of the sequence, where its chunks' states start
                                           // (only portions of several chunks keep states: at most 2 T / chunk of them)
 };
-__device__ __forceinline__ ChunkOf chunk_of(int index, const int* cu_q, int n_seqs, int chunk) {
+__device__ __forceinline__ ChunkOf chunk_of(int index, const int* cu_q, int n_seqs, int chunk, bool chunked) {
+    // (no portion longer than a chunk: chunk i is sequence i, and no walk over the sequences, whose every step
+    // would wait for a load)
+    if (!chunked) return ChunkOf{index < n_seqs ? index : -1, 0, 1, 0};
     ChunkOf c{0, index, 0, 0};
     for (; c.b < n_seqs; ++c.b) {
         c.n_chunks = max(1, (cu_q[c.b + 1] - cu_q[c.b] + chunk - 1) / chunk);
@@ -93,145 +97,238 @@ __device__ __forceinline__ ChunkOf chunk_of(int index, const int* cu_q, int n_se
     return c;
 }
 
-template <int NPT, int LANES_N>
+template <int NS>
 __global__ void __launch_bounds__(64)
 ssm_scan_kernel(const float* __restrict__ xbc, int ldx, const float* __restrict__ raw_dt, int ldd,
                 const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dskip,
                 const int* __restrict__ cu_q, const int* __restrict__ state_slots, int n_seqs, float* __restrict__ state,
-                size_t slot_floats, size_t scan_offset, float* __restrict__ y, int ldy, int H, int P, int N, int G,
-                int write, int chunk, float* __restrict__ chunk_state, float* __restrict__ cumlog) {
-    const int lane = threadIdx.x, ln = lane % LANES_N, pl = lane / LANES_N;
-    const int h = blockIdx.y;
-    const ChunkOf co = chunk_of(blockIdx.z, cu_q, n_seqs, chunk);
+                size_t slot_floats, size_t scan_offset, float* __restrict__ y, int ldy, size_t part_stride, int H, int P,
+                int N, int G, int n_slices, int write, int chunk, float* __restrict__ chunk_state,
+                float* __restrict__ cumlog) {
+    const int lane = threadIdx.x;
+    const int h = blockIdx.y, slice = blockIdx.x % n_slices, p = (blockIdx.x / n_slices) * 64 + lane;
+    const ChunkOf co = chunk_of(blockIdx.z, cu_q, n_seqs, chunk, chunk_state != nullptr);
     if (co.b < 0) return;                                      // surplus workgroup
     const int slot = state_slots[co.b];
     if (slot < 0) return;
-    const int p = blockIdx.x * (64 / LANES_N) + pl;
     const bool p_ok = p < P;
     const int pc = p_ok ? p : P - 1;
     const int g = h / (H / G), inner = H * P;
+    const int n0 = slice * NS, nn = min(NS, N - n0);
     const int t0 = cu_q[co.b] + co.k * chunk, t1 = min(t0 + chunk, cu_q[co.b + 1]);
-    float* sp = state + static_cast<size_t>(slot) * slot_floats + scan_offset + (static_cast<size_t>(h) * P + pc) * N;
-    float S[NPT];
+    float* sp = state + static_cast<size_t>(slot) * slot_floats + scan_offset + (static_cast<size_t>(h) * N + n0) * P + pc;
+    // (every load below is issued without a condition, from a clamped index, and masked by a select afterwards: a
+    // load under a condition waits for all loads in flight, which would make a token cost NS round trips)
+    float S[NS];
 #pragma unroll
-    for (int j = 0; j < NPT; ++j) {
-        const int n = j * LANES_N + ln;
-        S[j] = (co.k == 0 && n < N) ? sp[n] : 0.f;
-    }
-    const float bias = dt_bias[h], neg_rate = -expf(A_log[h]), skip = Dskip[h];
-    const int b_col = inner + g * N, c_col = inner + G * N + g * N;
-    // operands of the token at hand, and of the next one (loaded one token ahead)
-    float xv = 0.f, dtr = 0.f, Bv[NPT], Cv[NPT];
-    auto load = [&](int t, float& x_, float& d_, float (&B_)[NPT], float (&C_)[NPT]) {
-        const float* row = xbc + static_cast<size_t>(t) * ldx;
-        x_ = row[h * P + pc];
+    for (int j = 0; j < NS; ++j) S[j] = sp[static_cast<size_t>(min(j, nn - 1)) * P];
+#pragma unroll
+    for (int j = 0; j < NS; ++j) S[j] = (co.k == 0 && j < nn) ? S[j] : 0.f;
+    const float bias = dt_bias[h], neg_rate = -expf(A_log[h]), skip = slice == 0 ? Dskip[h] : 0.f;
+    const float* b_row = xbc + inner + g * N + n0;              // + t * ldx: B of the slice (the same for every lane)
+    const float* c_row = b_row + G * N;
+    float* yp = y + slice * part_stride + h * P + pc;
+    // a token's operands are requested one token ahead; rows of the slice beyond N count as zeros
+    float xv = 0.f, dtr = 0.f, Bv[NS], Cv[NS];
+    auto load = [&](int t, float& x_, float& d_, float (&B_)[NS], float (&C_)[NS]) {
+        x_ = xbc[static_cast<size_t>(t) * ldx + h * P + pc];
         d_ = raw_dt[static_cast<size_t>(t) * ldd + h];
+        const float* Bt = b_row + static_cast<size_t>(t) * ldx;
+        const float* Ct = c_row + static_cast<size_t>(t) * ldx;
 #pragma unroll
-        for (int j = 0; j < NPT; ++j) {
-            const int n = min(j * LANES_N + ln, N - 1);
-            B_[j] = row[b_col + n];
-            C_[j] = row[c_col + n];
+        for (int j = 0; j < NS; ++j) {
+            B_[j] = Bt[min(j, nn - 1)];
+            C_[j] = Ct[min(j, nn - 1)];
+        }
+#pragma unroll
+        for (int j = 0; j < NS; ++j) {
+            B_[j] = j < nn ? B_[j] : 0.f;
+            C_[j] = j < nn ? C_[j] : 0.f;
         }
     };
-    if (t0 < t1) load(t0, xv, dtr, Bv, Cv);
+    load(min(t0, t1 - 1), xv, dtr, Bv, Cv);
     float cum = 0.f;
     for (int t = t0; t < t1; ++t) {
-        float xn = 0.f, dn = 0.f, Bn[NPT], Cn[NPT];
-        const int tn = min(t + 1, t1 - 1);
-        load(tn, xn, dn, Bn, Cn);
+        float xn, dn, Bn[NS], Cn[NS];
+        load(min(t + 1, t1 - 1), xn, dn, Bn, Cn);
         const float dt = softplus_precise(dtr + bias);
         const float a = expf(neg_rate * dt), dx = dt * xv;
         cum += neg_rate * dt;
         float acc = 0.f;
 #pragma unroll
-        for (int j = 0; j < NPT; ++j) {
-            if (j * LANES_N + ln < N) {
-                S[j] = a * S[j] + dx * Bv[j];
-                acc += S[j] * Cv[j];
-            }
+        for (int j = 0; j < NS; ++j) {
+            S[j] = a * S[j] + dx * Bv[j];
+            acc += S[j] * Cv[j];
         }
-        acc = group_sum<LANES_N>(acc);
-        if (ln == 0 && p_ok) y[static_cast<size_t>(t) * ldy + h * P + p] = acc + skip * xv;
+        if (p_ok) yp[static_cast<size_t>(t) * ldy] = acc + skip * xv;
         if (co.n_chunks > 1 && blockIdx.x == 0 && lane == 0) cumlog[static_cast<size_t>(t) * H + h] = cum;
         xv = xn; dtr = dn;
 #pragma unroll
-        for (int j = 0; j < NPT; ++j) { Bv[j] = Bn[j]; Cv[j] = Cn[j]; }
+        for (int j = 0; j < NS; ++j) { Bv[j] = Bn[j]; Cv[j] = Cn[j]; }
     }
     if (!p_ok) return;
-    if (co.n_chunks > 1) sp = chunk_state + ((static_cast<size_t>(co.first_chunk + co.k) * H + h) * P + p) * N;
+    if (co.n_chunks > 1) sp = chunk_state + ((static_cast<size_t>(co.first_chunk + co.k) * H + h) * N + n0) * P + p;
     if (write || co.n_chunks > 1) {
 #pragma unroll
-        for (int j = 0; j < NPT; ++j) {
-            const int n = j * LANES_N + ln;
-            if (n < N) sp[n] = S[j];
+        for (int j = 0; j < NS; ++j)
+            if (j < nn) sp[static_cast<size_t>(j) * P] = S[j];
+    }
+}
+
+// The same scan with the chunk's operands staged in LDS first: x [chunk][64], B and C of the slice [chunk][NS]
+// and the raw step sizes, all requested at once with 16-byte loads, so that the token loop waits for no memory
+// (one token ahead is not enough to cover a load that another XCD's kernel wrote a moment ago). Needs 16-byte
+// aligned rows and column offsets (the launcher checks) and chunk <= CH.
+template <int NS, int CH>
+__global__ void __launch_bounds__(64)
+ssm_scan_staged_kernel(const float* __restrict__ xbc, int ldx, const float* __restrict__ raw_dt, int ldd,
+                       const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dskip,
+                       const int* __restrict__ cu_q, const int* __restrict__ state_slots, int n_seqs, float* __restrict__ state,
+                       size_t slot_floats, size_t scan_offset, float* __restrict__ y, int ldy, size_t part_stride, int H, int P,
+                       int N, int G, int n_slices, int write, int chunk, float* __restrict__ chunk_state,
+                       float* __restrict__ cumlog) {
+    __shared__ __attribute__((aligned(16))) float xs[CH][64];
+    __shared__ __attribute__((aligned(16))) float Bs[CH][NS];
+    __shared__ __attribute__((aligned(16))) float Cs[CH][NS];
+    __shared__ float dts[CH];
+    const int lane = threadIdx.x;
+    const int h = blockIdx.y, slice = blockIdx.x % n_slices, p0 = (blockIdx.x / n_slices) * 64, p = p0 + lane;
+    const ChunkOf co = chunk_of(blockIdx.z, cu_q, n_seqs, chunk, chunk_state != nullptr);
+    if (co.b < 0) return;
+    const int slot = state_slots[co.b];
+    if (slot < 0) return;
+    const bool p_ok = p < P;
+    const int pc = p_ok ? p : P - 1;
+    const int g = h / (H / G), inner = H * P;
+    const int n0 = slice * NS, nn = min(NS, N - n0);
+    const int t0 = cu_q[co.b] + co.k * chunk, t1 = min(t0 + chunk, cu_q[co.b + 1]), nt = t1 - t0;
+    float* sp = state + static_cast<size_t>(slot) * slot_floats + scan_offset + (static_cast<size_t>(h) * N + n0) * P + pc;
+    float S[NS];
+#pragma unroll
+    for (int j = 0; j < NS; ++j) S[j] = sp[static_cast<size_t>(min(j, nn - 1)) * P];
+    // staging: quads of 4 floats; a quad beyond the row's end (P or N no multiple of the tile) repeats the last one
+    const int pq = min(64, P - p0) / 4, nq = nn / 4;           // whole quads of x and of B, C in this tile
+    for (int e = lane; e < nt * 16; e += 64) {
+        const int tt = e / 16, q = min(e % 16, pq - 1);
+        *reinterpret_cast<float4*>(&xs[tt][4 * (e % 16)]) =
+            *reinterpret_cast<const float4*>(xbc + static_cast<size_t>(t0 + tt) * ldx + h * P + p0 + 4 * q);
+    }
+    for (int e = lane; e < nt * (NS / 4); e += 64) {
+        const int tt = e / (NS / 4), qi = e % (NS / 4), q = min(qi, nq - 1);
+        const float* row = xbc + static_cast<size_t>(t0 + tt) * ldx + inner + g * N + n0 + 4 * q;
+        float4 bq = *reinterpret_cast<const float4*>(row), cq = *reinterpret_cast<const float4*>(row + G * N);
+        if (qi >= nq) { bq = make_float4(0.f, 0.f, 0.f, 0.f); cq = bq; }          // rows of the slice beyond N count as zeros
+        *reinterpret_cast<float4*>(&Bs[tt][4 * qi]) = bq;
+        *reinterpret_cast<float4*>(&Cs[tt][4 * qi]) = cq;
+    }
+    if (lane < nt) dts[lane] = raw_dt[static_cast<size_t>(t0 + lane) * ldd + h];
+#pragma unroll
+    for (int j = 0; j < NS; ++j) S[j] = (co.k == 0 && j < nn) ? S[j] : 0.f;
+    const float bias = dt_bias[h], neg_rate = -expf(A_log[h]), skip = slice == 0 ? Dskip[h] : 0.f;
+    float* yp = y + slice * part_stride + h * P + pc;
+    wave_lds_sync();
+    float cum = 0.f;
+    for (int tt = 0; tt < nt; ++tt) {
+        const float xv = xs[tt][lane];
+        const float dt = softplus_precise(dts[tt] + bias);
+        const float a = expf(neg_rate * dt), dx = dt * xv;
+        cum += neg_rate * dt;
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < NS; j += 4) {
+            const float4 b4 = *reinterpret_cast<const float4*>(&Bs[tt][j]), c4 = *reinterpret_cast<const float4*>(&Cs[tt][j]);
+            S[j] = a * S[j] + dx * b4.x;         acc += S[j] * c4.x;
+            S[j + 1] = a * S[j + 1] + dx * b4.y; acc += S[j + 1] * c4.y;
+            S[j + 2] = a * S[j + 2] + dx * b4.z; acc += S[j + 2] * c4.z;
+            S[j + 3] = a * S[j + 3] + dx * b4.w; acc += S[j + 3] * c4.w;
         }
+        if (p_ok) yp[static_cast<size_t>(t0 + tt) * ldy] = acc + skip * xv;
+        if (co.n_chunks > 1 && blockIdx.x == 0 && lane == 0) cumlog[static_cast<size_t>(t0 + tt) * H + h] = cum;
+    }
+    if (!p_ok) return;
+    if (co.n_chunks > 1) sp = chunk_state + ((static_cast<size_t>(co.first_chunk + co.k) * H + h) * N + n0) * P + p;
+    if (write || co.n_chunks > 1) {
+#pragma unroll
+        for (int j = 0; j < NS; ++j)
+            if (j < nn) sp[static_cast<size_t>(j) * P] = S[j];
     }
 }
 
 // What the chunks before chunk k of a portion contribute to it (see ssm_scan_kernel): with A_j the whole
 // decay of chunk j and L_j its last local state, the state at the start of chunk k is
 //   S = L_0 for k = 1;  S <- A_j S + L_j for j = 1 .. k - 1,
-// every token t of chunk k gets  y[t] += exp(cumlog[t]) sum_n C[t, n] S[n, p], and the portion's last chunk
-// writes A_k S + L_k back to the slot. Same grid and lane layout as the scan.
-template <int NPT, int LANES_N>
+// every token t of chunk k gets  y[t] += exp(cumlog[t]) sum_n C[t, n] S[n, p] (slice by slice, as the scan), and
+// the portion's last chunk writes A_k S + L_k back to the slot. Same grid and lane layout as the scan.
+template <int NS>
 __global__ void __launch_bounds__(64)
 ssm_chunk_join_kernel(const float* __restrict__ xbc, int ldx, const int* __restrict__ cu_q, const int* __restrict__ state_slots,
                       int n_seqs, float* __restrict__ state, size_t slot_floats, size_t scan_offset, float* __restrict__ y,
-                      int ldy, int H, int P, int N, int G, int write, int chunk, const float* __restrict__ chunk_state,
-                      const float* __restrict__ cumlog) {
-    const int lane = threadIdx.x, ln = lane % LANES_N, pl = lane / LANES_N;
-    const int h = blockIdx.y;
-    const ChunkOf co = chunk_of(blockIdx.z, cu_q, n_seqs, chunk);
+                      int ldy, size_t part_stride, int H, int P, int N, int G, int n_slices, int write, int chunk,
+                      const float* __restrict__ chunk_state, const float* __restrict__ cumlog) {
+    const int lane = threadIdx.x;
+    const int h = blockIdx.y, slice = blockIdx.x % n_slices, p = (blockIdx.x / n_slices) * 64 + lane;
+    const ChunkOf co = chunk_of(blockIdx.z, cu_q, n_seqs, chunk, true);
     if (co.b < 0 || co.k == 0) return;                         // surplus, or a first chunk: nothing comes before it
     const int slot = state_slots[co.b];
     if (slot < 0) return;
-    const int p = blockIdx.x * (64 / LANES_N) + pl;
     const bool p_ok = p < P;
     const int pc = p_ok ? p : P - 1;
     const int g = h / (H / G), inner = H * P;
+    const int n0 = slice * NS, nn = min(NS, N - n0);
     const int q0 = cu_q[co.b], q1 = cu_q[co.b + 1];
-    auto local_state = [&](int j) { return chunk_state + ((static_cast<size_t>(co.first_chunk + j) * H + h) * P + pc) * N; };
+    auto local_state = [&](int j) { return chunk_state + ((static_cast<size_t>(co.first_chunk + j) * H + h) * N + n0) * P + pc; };
     auto chunk_decay = [&](int j) { return expf(cumlog[static_cast<size_t>(min(q0 + (j + 1) * chunk, q1) - 1) * H + h]); };
-    float S[NPT];
+    // (loads without conditions, from clamped indices, as in the scan; rows of the slice beyond N stay zero)
+    float S[NS];
     {
         const float* l0 = local_state(0);
 #pragma unroll
-        for (int j = 0; j < NPT; ++j) {
-            const int n = j * LANES_N + ln;
-            S[j] = n < N ? l0[n] : 0.f;
-        }
+        for (int j = 0; j < NS; ++j) S[j] = l0[static_cast<size_t>(min(j, nn - 1)) * P];
+#pragma unroll
+        for (int j = 0; j < NS; ++j) S[j] = j < nn ? S[j] : 0.f;
     }
     for (int c = 1; c < co.k; ++c) {
         const float a = chunk_decay(c);
         const float* lc = local_state(c);
+        float L[NS];
 #pragma unroll
-        for (int j = 0; j < NPT; ++j) {
-            const int n = j * LANES_N + ln;
-            if (n < N) S[j] = a * S[j] + lc[n];
-        }
+        for (int j = 0; j < NS; ++j) L[j] = lc[static_cast<size_t>(min(j, nn - 1)) * P];
+#pragma unroll
+        for (int j = 0; j < NS; ++j) S[j] = j < nn ? a * S[j] + L[j] : 0.f;
     }
     const int t0 = q0 + co.k * chunk, t1 = min(t0 + chunk, q1);
-    const int c_col = inner + G * N + g * N;
-    for (int t = t0; t < t1; ++t) {
-        const float* row = xbc + static_cast<size_t>(t) * ldx;
-        float acc = 0.f;
+    const float* c_row = xbc + inner + G * N + g * N + n0;
+    float* yp = y + slice * part_stride + h * P + pc;
+    // eight tokens at a time: their C rows, decays and y values are requested together, then used
+    for (int t = t0; t < t1; t += 8) {
+        float Cv[8][NS], seen[8], before[8];
 #pragma unroll
-        for (int j = 0; j < NPT; ++j) {
-            const int n = j * LANES_N + ln;
-            if (n < N) acc += S[j] * row[c_col + n];
+        for (int u = 0; u < 8; ++u) {
+            const int tu = min(t + u, t1 - 1);
+            const float* Ct = c_row + static_cast<size_t>(tu) * ldx;
+#pragma unroll
+            for (int j = 0; j < NS; ++j) Cv[u][j] = Ct[min(j, nn - 1)];
+            seen[u] = cumlog[static_cast<size_t>(tu) * H + h];
+            before[u] = yp[static_cast<size_t>(tu) * ldy];          // (pc is a valid column for every lane)
         }
-        acc = group_sum<LANES_N>(acc);
-        if (ln == 0 && p_ok) y[static_cast<size_t>(t) * ldy + h * P + p] += expf(cumlog[static_cast<size_t>(t) * H + h]) * acc;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < NS; ++j) acc += S[j] * Cv[u][j];     // (S is zero beyond N)
+            if (p_ok && t + u < t1) yp[static_cast<size_t>(t + u) * ldy] = before[u] + expf(seen[u]) * acc;
+        }
     }
-    if (write && p_ok && co.k == co.n_chunks - 1) {
+    if (write && co.k == co.n_chunks - 1) {
         const float a = chunk_decay(co.k);
         const float* lk = local_state(co.k);
-        float* sp = state + static_cast<size_t>(slot) * slot_floats + scan_offset + (static_cast<size_t>(h) * P + p) * N;
+        float L[NS];
 #pragma unroll
-        for (int j = 0; j < NPT; ++j) {
-            const int n = j * LANES_N + ln;
-            if (n < N) sp[n] = a * S[j] + lk[n];
-        }
+        for (int j = 0; j < NS; ++j) L[j] = lk[static_cast<size_t>(min(j, nn - 1)) * P];
+        float* sp = state + static_cast<size_t>(slot) * slot_floats + scan_offset + (static_cast<size_t>(h) * N + n0) * P + pc;
+#pragma unroll
+        for (int j = 0; j < NS; ++j)
+            if (j < nn && p_ok) sp[static_cast<size_t>(j) * P] = a * S[j] + L[j];
     }
 }
 
@@ -260,51 +357,47 @@ int mllm_conv_silu(const float* proj, int ld, int col0, int C, const float* w, c
     return 0;
 }
 
-// Tokens of a chunk, and what the chunks' workspace must hold for a step of T tokens in B sequences.
+// Tokens of a chunk, rows of n a wavefront keeps, and what the chunks' workspace must hold for a step of T tokens.
 #define SSM_CHUNK 64
+#define SSM_SLICE 32
 static size_t chunk_states(int T) { return 2 * static_cast<size_t>(T) / SSM_CHUNK + 1; }
 size_t mllm_ssm_scan_workspace_floats(int T, int B, int H, int P, int N) {
     (void)B;
     return chunk_states(T) * H * P * N + static_cast<size_t>(T) * H;
 }
+// The scan leaves y as this many shares (see ssm_scan_kernel), part_stride floats apart.
+int mllm_ssm_scan_parts(int N) { return (N + SSM_SLICE - 1) / SSM_SLICE; }
 
 // The scan over every sequence's portion (see the kernels). `workspace` (mllm_ssm_scan_workspace_floats floats)
-// is needed when a portion is longer than one chunk (max_q_len > 64). -1: H is no multiple of G, N > 1024, or
-// the workspace is missing.
+// is needed when a portion is longer than one chunk (max_q_len > 64). -1: H is no multiple of G, or the
+// workspace is missing.
 int mllm_ssm_scan(const float* xbc, int ldx, const float* raw_dt, int ldd, const float* dt_bias, const float* A_log,
                   const float* Dskip, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
-                  size_t scan_offset, float* y, int ldy, int T, int B, int max_q_len, int H, int P, int N, int G, int write,
-                  float* workspace, hipStream_t stream) {
+                  size_t scan_offset, float* y, int ldy, size_t part_stride, int T, int B, int max_q_len, int H, int P, int N,
+                  int G, int write, float* workspace, hipStream_t stream) {
     if (B <= 0 || T <= 0) return 0;
-    if (H < 1 || G < 1 || H % G != 0 || N < 1 || N > 1024 || P < 1) return -1;
+    if (H < 1 || G < 1 || H % G != 0 || N < 1 || P < 1) return -1;
     const bool chunked = max_q_len > SSM_CHUNK;
     if (chunked && workspace == nullptr) return -1;
     const int n_chunks = chunked ? T / SSM_CHUNK + B : B;
     float* chunk_state = workspace;
     float* cumlog = workspace ? workspace + chunk_states(T) * H * P * N : nullptr;
-    int lanes = 1;
-    while (lanes < 64 && lanes * 16 < N) lanes *= 2;       // sixteen n a lane
-#define SCAN(L)                                                                                                       \
-    do {                                                                                                              \
-        const dim3 grid((P + 64 / L - 1) / (64 / L), H, n_chunks);                                                    \
-        ssm_scan_kernel<16, L><<<grid, 64, 0, stream>>>(xbc, ldx, raw_dt, ldd, dt_bias, A_log, Dskip, cu_q, state_slots, B, \
-                                                        state, slot_floats, scan_offset, y, ldy, H, P, N, G, write,   \
-                                                        SSM_CHUNK, chunk_state, cumlog);                              \
-        if (chunked)                                                                                                  \
-            ssm_chunk_join_kernel<16, L><<<grid, 64, 0, stream>>>(xbc, ldx, cu_q, state_slots, B, state, slot_floats, \
-                                                                  scan_offset, y, ldy, H, P, N, G, write, SSM_CHUNK,  \
-                                                                  chunk_state, cumlog);                               \
-    } while (0)
-    switch (lanes) {
-        case 1: SCAN(1); break;
-        case 2: SCAN(2); break;
-        case 4: SCAN(4); break;
-        case 8: SCAN(8); break;
-        case 16: SCAN(16); break;
-        case 32: SCAN(32); break;
-        default: SCAN(64); break;
-    }
-#undef SCAN
+    const int n_slices = mllm_ssm_scan_parts(N);
+    const dim3 grid(((P + 63) / 64) * n_slices, H, n_chunks);
+    const bool aligned = ldx % 4 == 0 && P % 4 == 0 && N % 4 == 0 && (reinterpret_cast<uintptr_t>(xbc) & 15) == 0;
+    if (aligned)
+        ssm_scan_staged_kernel<SSM_SLICE, SSM_CHUNK><<<grid, 64, 0, stream>>>(xbc, ldx, raw_dt, ldd, dt_bias, A_log, Dskip, cu_q, state_slots,
+                                                                             B, state, slot_floats, scan_offset, y, ldy, part_stride, H, P, N,
+                                                                             G, n_slices, write, SSM_CHUNK, chunked ? chunk_state : nullptr,
+                                                                             cumlog);
+    else
+        ssm_scan_kernel<SSM_SLICE><<<grid, 64, 0, stream>>>(xbc, ldx, raw_dt, ldd, dt_bias, A_log, Dskip, cu_q, state_slots, B, state,
+                                                           slot_floats, scan_offset, y, ldy, part_stride, H, P, N, G, n_slices, write,
+                                                           SSM_CHUNK, chunked ? chunk_state : nullptr, cumlog);
+    if (chunked)
+        ssm_chunk_join_kernel<SSM_SLICE><<<grid, 64, 0, stream>>>(xbc, ldx, cu_q, state_slots, B, state, slot_floats, scan_offset, y,
+                                                                 ldy, part_stride, H, P, N, G, n_slices, write, SSM_CHUNK,
+                                                                 chunk_state, cumlog);
     MLLM_LAUNCH_CHECK();
     return 0;
 }
