@@ -22,6 +22,8 @@ int mllm_kv_append(const void* src, int src_stride, int k_col, int v_col, void* 
 // gemm_f32.hip, gemm_bf16.hip
 int mllm_gemm_f32(const float* A, int lda, const float* W, int ldw, const float* bias, void* C, int ldc,
                   int M, int N, int K, int mode, hipStream_t stream);
+int mllm_gemm_bf16_plain(const void* A, int lda, const void* W, int ldw, const float* bias, void* C, int ldc,
+                         int M, int N, int K, int mode, hipStream_t stream);
 int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C, int ldc,
                    int M, int N, int K, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream);
 int mllm_gemm_bf16_kv(const void* A, int lda, const void* W, int ldw, const float* bias, void* C, int ldc,

@@ -255,6 +255,10 @@ void linear(const Tensor2& a, const Tensor2& w, const float* bias, const Tensor2
         rc = mllm_gemm_f32(static_cast<const float*>(a.data), static_cast<int>(a.stride), static_cast<const float*>(w.data),
                            static_cast<int>(w.stride), bias, out.data, static_cast<int>(out.stride), static_cast<int>(M),
                            static_cast<int>(N), static_cast<int>(K), epilogue, stream);
+    } else if (kv == nullptr && (K % 8 != 0 || a.stride % 8 != 0 || w.stride % 8 != 0 || !aligned(a.data, 16) || !aligned(w.data, 16))) {
+        // sizes that the matrix-core kernels do not read (16 bytes at a time): the plain kernel, slow and general
+        rc = mllm_gemm_bf16_plain(a.data, static_cast<int>(a.stride), w.data, static_cast<int>(w.stride), bias, out.data,
+                                  static_cast<int>(out.stride), static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), epilogue, stream);
     } else if (kv != nullptr) {
         rc = mllm_gemm_bf16_kv(a.data, static_cast<int>(a.stride), w.data, static_cast<int>(w.stride), bias, out.data,
                                static_cast<int>(out.stride), static_cast<int>(M), static_cast<int>(N), static_cast<int>(K),
@@ -306,7 +310,7 @@ void ln_linear(const Tensor2& x, const float* gamma, const float* beta, float ep
     // (More rows than that: the norm is a kernel of its own. Normalising in the tiled product while it stages
     // its rows was measured at 64 to 256 rows and lost: every workgroup of a row tile has to pull the tile's
     // fp32 rows through its own L1 for the statistics, 6.5 us at 64 rows of 768, more than the norm's kernel.)
-    if (kv == nullptr && w.dtype == BF16 && M <= tuning().ln_fuse_max_rows && x.contiguous() && aligned(gamma, 16) &&
+    if (kv == nullptr && w.dtype == BF16 && K % 8 == 0 && w.stride % 8 == 0 && M <= tuning().ln_fuse_max_rows && x.contiguous() && aligned(gamma, 16) &&
         (beta == nullptr || aligned(beta, 16))) {
         const int rc = mllm_ln_gemm_bf16(static_cast<const float*>(x.data), static_cast<int>(x.stride), rows, gamma, beta, eps,
                                          w.data, static_cast<int>(w.stride), bias, out.data, static_cast<int>(out.stride),

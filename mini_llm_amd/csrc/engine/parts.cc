@@ -92,10 +92,8 @@ const Tensor2* Params::weights_or_null(const std::string& key) const {
 }
 
 Linear::Linear(const Tensor2& w, const Tensor2* b) : weight(w) {
-    // (said when the model is built, not at its first step: the bfloat16 products read 16 bytes at a time)
-    if (w.dtype == BF16 && (w.cols % 8 != 0 || w.stride % 8 != 0))
-        fail("a linear map of %lld inputs has no bfloat16 kernel: the number of inputs must be a multiple of 8 (float32 takes any)",
-             (long long)w.cols);
+    // (any number of inputs: the bfloat16 matrix-core kernels read 16 bytes at a time, and a map whose inputs are
+    // no multiple of 8 goes to a plain kernel instead)
     if (b != nullptr) {
         if (b->dtype != F32 || b->rows * b->cols != w.rows || !b->contiguous())
             fail("a linear map's bias must be contiguous float32 [%lld]", (long long)w.rows);

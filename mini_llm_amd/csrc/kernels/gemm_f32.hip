@@ -7,6 +7,8 @@
 // Same contract as the reference's bounds-safe kernel
 // (/root/reference/src/kernels/gemm.cu:238-392: alpha*acc + beta*old + bias, optional GELU),
 // with the weight held as [N,K] (k contiguous) instead of [K,N].
+#include <algorithm>
+
 #include "common.h"
 
 #define F32_BM 64
@@ -165,7 +167,41 @@ gemm_f32_rows_kernel(const float* __restrict__ A, int lda, const float* __restri
     }
 }
 
+// bfloat16 operands of any K, strides and alignment (what the matrix-core kernels of gemm_bf16.hip refuse:
+// they read 16 bytes at a time): one wavefront per output column and 8 rows, the lanes over k, sums in fp32.
+__global__ void __launch_bounds__(256)
+gemm_bf16_plain_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
+                       const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
+    const int n = blockIdx.x * 4 + wave;
+    if (n >= N) return;
+    const bf16_t* wr = W + static_cast<size_t>(n) * ldw;
+    for (int m0 = blockIdx.y * 8; m0 < M; m0 += gridDim.y * 8) {
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int k = lane; k < K; k += 64) {
+            const float wv = to_float(wr[k]);
+#pragma unroll
+            for (int r = 0; r < 8; ++r) acc[r] += wv * to_float(A[static_cast<size_t>(min(m0 + r, M - 1)) * lda + k]);
+        }
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const float v = wave_sum(acc[r]);
+            if (lane == 0 && m0 + r < M) epilogue<bf16_t>(mode, v, bias ? bias[n] : 0.f, C, static_cast<size_t>(m0 + r) * ldc + n);
+        }
+    }
+}
+
 extern "C" {
+
+int mllm_gemm_bf16_plain(const void* A, int lda, const void* W, int ldw, const float* bias, void* C, int ldc,
+                         int M, int N, int K, int mode, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    const dim3 grid((N + 3) / 4, std::min((M + 7) / 8, 256));
+    gemm_bf16_plain_kernel<<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), ldw, bias, C, ldc,
+                                                     M, N, K, mode);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
 
 int mllm_gemm_f32(const float* A, int lda, const float* W, int ldw, const float* bias, void* C, int ldc,
                   int M, int N, int K, int mode, hipStream_t stream) {

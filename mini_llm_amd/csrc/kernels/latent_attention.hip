@@ -375,25 +375,42 @@ latent_prefill_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ 
         kt_begin += static_cast<int>(blockIdx.y) * per;
         kt_end = min(kt_end, kt_begin + per);
     }
+    static_assert(DT % 2 == 0, "the transposed latent is staged in whole rounds of the workgroup");
     for (int kt = kt_begin; kt < kt_end; ++kt) {
         const int j_base = kt * BN;
-        __syncthreads();                           // the tile before is used up
-        // page rows, row-major; a key outside [k_lo, p_last] is replaced by one inside (always a held page;
-        // its scores are masked below)
-        for (int idx = tid; idx < BN * CH; idx += 256) {
-            const int j = idx / CH, c = idx % CH;
+        // Staging. All loads of a tile are issued first (a fixed number per thread: 64 * E / 8 pieces of page rows
+        // over 256 threads are KS each, R * 8 pieces of the transposed latent DT / 2 each), then written to LDS: a
+        // load inside a loop of unknown length would be waited for before the next one is asked for.
+        // Page rows, row-major; a key outside [k_lo, p_last] is replaced by one inside (always a held page; its
+        // scores are masked below). The latent transposed: 8 keys of one column a piece, keys outside the range
+        // set to zero.
+        u32x4 kreg[KS], vreg[DT / 2];
+#pragma unroll
+        for (int u = 0; u < KS; ++u) {
+            const int idx = tid + 256 * u, j = idx / CH, c = idx % CH;
             const int key = min(max(j_base + j, k_lo), p_last);
             const size_t row = (static_cast<size_t>(sm_table[key >> shift]) << shift) + (key & (page_size - 1));
-            *reinterpret_cast<u32x4*>(Ks + j * KSTRIDE + 8 * c) = *reinterpret_cast<const u32x4*>(k_pages + row * E + 8 * c);
+            kreg[u] = *reinterpret_cast<const u32x4*>(k_pages + row * E + 8 * c);
         }
-        // the latent transposed: 8 keys of one column a piece
-        for (int idx = tid; idx < R * (BN / 8); idx += 256) {
-            const int col = idx / (BN / 8), part = idx % (BN / 8);
+#pragma unroll
+        for (int u = 0; u < DT / 2; ++u) {
+            const int idx = tid + 256 * u, col = idx / (BN / 8), part = idx % (BN / 8);
             const int key0 = j_base + 8 * part;
             const int pg = min(max(key0 >> shift, pg_lo), pg_hi);
-            const bf16_t* src = vt_pages + (static_cast<size_t>(sm_table[pg]) << shift) * R + static_cast<size_t>(col) * page_size +
-                                (key0 & (page_size - 1));
-            u32x4 v = *reinterpret_cast<const u32x4*>(src);
+            vreg[u] = *reinterpret_cast<const u32x4*>(vt_pages + (static_cast<size_t>(sm_table[pg]) << shift) * R +
+                                                      static_cast<size_t>(col) * page_size + (key0 & (page_size - 1)));
+        }
+        __syncthreads();                           // the tile before is used up
+#pragma unroll
+        for (int u = 0; u < KS; ++u) {
+            const int idx = tid + 256 * u, j = idx / CH, c = idx % CH;
+            *reinterpret_cast<u32x4*>(Ks + j * KSTRIDE + 8 * c) = kreg[u];
+        }
+#pragma unroll
+        for (int u = 0; u < DT / 2; ++u) {
+            const int idx = tid + 256 * u, col = idx / (BN / 8), part = idx % (BN / 8);
+            const int key0 = j_base + 8 * part;
+            u32x4 v = vreg[u];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int ka = key0 + 2 * e, kb = ka + 1;

@@ -190,7 +190,7 @@ ssm_scan_staged_kernel(const float* __restrict__ xbc, int ldx, const float* __re
     __shared__ __attribute__((aligned(16))) float xs[CH][64];
     __shared__ __attribute__((aligned(16))) float Bs[CH][NS];
     __shared__ __attribute__((aligned(16))) float Cs[CH][NS];
-    __shared__ float dts[CH];
+    __shared__ float dts[64], as[64];                 // step size and decay of the chunk's tokens
     const int lane = threadIdx.x;
     const int h = blockIdx.y, slice = blockIdx.x % n_slices, p0 = (blockIdx.x / n_slices) * 64, p = p0 + lane;
     const ChunkOf co = chunk_of(blockIdx.z, cu_q, n_seqs, chunk, chunk_state != nullptr);
@@ -206,44 +206,74 @@ ssm_scan_staged_kernel(const float* __restrict__ xbc, int ldx, const float* __re
     float S[NS];
 #pragma unroll
     for (int j = 0; j < NS; ++j) S[j] = sp[static_cast<size_t>(min(j, nn - 1)) * P];
-    // staging: quads of 4 floats; a quad beyond the row's end (P or N no multiple of the tile) repeats the last one
+    // Staging: quads of 4 floats, a fixed number per lane (CH * 16 quads of x, CH * NS / 4 of B and of C over 64
+    // lanes), all requested before the first is written to LDS; tokens beyond the chunk's end repeat its last one,
+    // a quad beyond the row's end (P or N no multiple of the tile) the row's last one.
     const int pq = min(64, P - p0) / 4, nq = nn / 4;           // whole quads of x and of B, C in this tile
-    for (int e = lane; e < nt * 16; e += 64) {
-        const int tt = e / 16, q = min(e % 16, pq - 1);
-        *reinterpret_cast<float4*>(&xs[tt][4 * (e % 16)]) =
-            *reinterpret_cast<const float4*>(xbc + static_cast<size_t>(t0 + tt) * ldx + h * P + p0 + 4 * q);
+    {
+        float4 xq[CH / 4];
+#pragma unroll
+        for (int u = 0; u < CH / 4; ++u) {
+            const int e = lane + 64 * u, tt = min(e / 16, nt - 1), q = min(e % 16, pq - 1);
+            xq[u] = *reinterpret_cast<const float4*>(xbc + static_cast<size_t>(t0 + tt) * ldx + h * P + p0 + 4 * q);
+        }
+        constexpr int BQ = CH * (NS / 4) / 64;
+        float4 bq[BQ], cq[BQ];
+#pragma unroll
+        for (int u = 0; u < BQ; ++u) {
+            const int e = lane + 64 * u, tt = min(e / (NS / 4), nt - 1), q = min(e % (NS / 4), nq - 1);
+            const float* row = xbc + static_cast<size_t>(t0 + tt) * ldx + inner + g * N + n0 + 4 * q;
+            bq[u] = *reinterpret_cast<const float4*>(row);
+            cq[u] = *reinterpret_cast<const float4*>(row + G * N);
+        }
+#pragma unroll
+        for (int u = 0; u < CH / 4; ++u) {
+            const int e = lane + 64 * u;
+            *reinterpret_cast<float4*>(&xs[e / 16][4 * (e % 16)]) = xq[u];
+        }
+#pragma unroll
+        for (int u = 0; u < BQ; ++u) {
+            const int e = lane + 64 * u, qi = e % (NS / 4);
+            const bool real = qi < nq;                          // rows of the slice beyond N count as zeros
+            *reinterpret_cast<float4*>(&Bs[e / (NS / 4)][4 * qi]) = real ? bq[u] : make_float4(0.f, 0.f, 0.f, 0.f);
+            *reinterpret_cast<float4*>(&Cs[e / (NS / 4)][4 * qi]) = real ? cq[u] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
     }
-    for (int e = lane; e < nt * (NS / 4); e += 64) {
-        const int tt = e / (NS / 4), qi = e % (NS / 4), q = min(qi, nq - 1);
-        const float* row = xbc + static_cast<size_t>(t0 + tt) * ldx + inner + g * N + n0 + 4 * q;
-        float4 bq = *reinterpret_cast<const float4*>(row), cq = *reinterpret_cast<const float4*>(row + G * N);
-        if (qi >= nq) { bq = make_float4(0.f, 0.f, 0.f, 0.f); cq = bq; }          // rows of the slice beyond N count as zeros
-        *reinterpret_cast<float4*>(&Bs[tt][4 * qi]) = bq;
-        *reinterpret_cast<float4*>(&Cs[tt][4 * qi]) = cq;
+    // Step sizes and decays are the same for every lane: lane t works them out for token t of the chunk, once
+    // (softplus, two exponentials), and a running sum over the lanes gives the logarithm of the decay accumulated
+    // since the chunk began.
+    const float bias = dt_bias[h], neg_rate = -expf(A_log[h]), skip = slice == 0 ? Dskip[h] : 0.f;
+    {
+        static_assert(CH <= 64, "one lane per token of a chunk");
+        const float dt = softplus_precise(raw_dt[static_cast<size_t>(t0 + min(lane, nt - 1)) * ldd + h] + bias);
+        const float lg = lane < nt ? neg_rate * dt : 0.f;
+        float run = lg;
+#pragma unroll
+        for (int off = 1; off < 64; off *= 2) {
+            const float up = __shfl_up(run, off, 64);
+            if (lane >= off) run += up;
+        }
+        dts[lane] = dt;
+        as[lane] = expf(lg);
+        if (co.n_chunks > 1 && blockIdx.x == 0 && lane < nt) cumlog[static_cast<size_t>(t0 + lane) * H + h] = run;
     }
-    if (lane < nt) dts[lane] = raw_dt[static_cast<size_t>(t0 + lane) * ldd + h];
 #pragma unroll
     for (int j = 0; j < NS; ++j) S[j] = (co.k == 0 && j < nn) ? S[j] : 0.f;
-    const float bias = dt_bias[h], neg_rate = -expf(A_log[h]), skip = slice == 0 ? Dskip[h] : 0.f;
     float* yp = y + slice * part_stride + h * P + pc;
     wave_lds_sync();
-    float cum = 0.f;
     for (int tt = 0; tt < nt; ++tt) {
         const float xv = xs[tt][lane];
-        const float dt = softplus_precise(dts[tt] + bias);
-        const float a = expf(neg_rate * dt), dx = dt * xv;
-        cum += neg_rate * dt;
-        float acc = 0.f;
+        const float a = as[tt], dx = dts[tt] * xv;
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < NS; j += 4) {
             const float4 b4 = *reinterpret_cast<const float4*>(&Bs[tt][j]), c4 = *reinterpret_cast<const float4*>(&Cs[tt][j]);
-            S[j] = a * S[j] + dx * b4.x;         acc += S[j] * c4.x;
-            S[j + 1] = a * S[j + 1] + dx * b4.y; acc += S[j + 1] * c4.y;
-            S[j + 2] = a * S[j + 2] + dx * b4.z; acc += S[j + 2] * c4.z;
-            S[j + 3] = a * S[j + 3] + dx * b4.w; acc += S[j + 3] * c4.w;
+            S[j] = a * S[j] + dx * b4.x;         acc[0] += S[j] * c4.x;
+            S[j + 1] = a * S[j + 1] + dx * b4.y; acc[1] += S[j + 1] * c4.y;
+            S[j + 2] = a * S[j + 2] + dx * b4.z; acc[2] += S[j + 2] * c4.z;
+            S[j + 3] = a * S[j + 3] + dx * b4.w; acc[3] += S[j + 3] * c4.w;
         }
-        if (p_ok) yp[static_cast<size_t>(t0 + tt) * ldy] = acc + skip * xv;
-        if (co.n_chunks > 1 && blockIdx.x == 0 && lane == 0) cumlog[static_cast<size_t>(t0 + tt) * H + h] = cum;
+        if (p_ok) yp[static_cast<size_t>(t0 + tt) * ldy] = (acc[0] + acc[1]) + (acc[2] + acc[3]) + skip * xv;
     }
     if (!p_ok) return;
     if (co.n_chunks > 1) sp = chunk_state + ((static_cast<size_t>(co.first_chunk + co.k) * H + h) * N + n0) * P + p;
@@ -299,24 +329,38 @@ ssm_chunk_join_kernel(const float* __restrict__ xbc, int ldx, const int* __restr
     const int t0 = q0 + co.k * chunk, t1 = min(t0 + chunk, q1);
     const float* c_row = xbc + inner + G * N + g * N + n0;
     float* yp = y + slice * part_stride + h * P + pc;
-    // eight tokens at a time: their C rows, decays and y values are requested together, then used
-    for (int t = t0; t < t1; t += 8) {
-        float Cv[8][NS], seen[8], before[8];
+    // the chunk's C rows of the slice and its tokens' decays go to LDS first, all requested at once (as the scan
+    // stages its operands); y is then read, added to and written sixteen tokens at a time
+    __shared__ float Cs[64][NS + 1];
+    __shared__ float seen_s[64];
+    const int nt = t1 - t0;
+    {
+        float cv[NS];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int tu = min(t + u, t1 - 1);
-            const float* Ct = c_row + static_cast<size_t>(tu) * ldx;
-#pragma unroll
-            for (int j = 0; j < NS; ++j) Cv[u][j] = Ct[min(j, nn - 1)];
-            seen[u] = cumlog[static_cast<size_t>(tu) * H + h];
-            before[u] = yp[static_cast<size_t>(tu) * ldy];          // (pc is a valid column for every lane)
+        for (int u = 0; u < NS; ++u) {
+            const int e = lane + 64 * u, tt = min(e / NS, nt - 1), j = min(e % NS, nn - 1);
+            cv[u] = c_row[static_cast<size_t>(t0 + tt) * ldx + j];
         }
+        const float sv = cumlog[static_cast<size_t>(t0 + min(lane, nt - 1)) * H + h];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < NS; ++u) {
+            const int e = lane + 64 * u;
+            Cs[e / NS][e % NS] = cv[u];
+        }
+        seen_s[lane] = expf(sv);
+    }
+    wave_lds_sync();
+    for (int t = 0; t < nt; t += 16) {
+        float before[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) before[u] = yp[static_cast<size_t>(t0 + min(t + u, nt - 1)) * ldy];     // (pc is a valid column for every lane)
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int tt = min(t + u, nt - 1);
             float acc = 0.f;
 #pragma unroll
-            for (int j = 0; j < NS; ++j) acc += S[j] * Cv[u][j];     // (S is zero beyond N)
-            if (p_ok && t + u < t1) yp[static_cast<size_t>(t + u) * ldy] = before[u] + expf(seen[u]) * acc;
+            for (int j = 0; j < NS; ++j) acc += S[j] * Cs[tt][j];         // (S is zero beyond N)
+            if (p_ok && t + u < nt) yp[static_cast<size_t>(t0 + t + u) * ldy] = before[u] + seen_s[tt] * acc;
         }
     }
     if (write && co.k == co.n_chunks - 1) {

@@ -66,6 +66,14 @@ TILED = model([
     latent(heads=2, dim=24, rot_dim=32, vdim=8, kv_rank=128, q_rank=16, window=70, kv_from=2),
 ], vocab=211, width=56, mult=0.6)
 
+# sizes that are multiples of neither 8 nor 4: the plain bfloat16 product, the scan without staging, rows of the
+# pages that are not 16-byte pieces
+ODD = model([
+    mamba(heads=3, vdim=12, state=10, groups=1, conv=2, norm_groups=3, mlp=dense(52, 1.0)),
+    latent(heads=3, dim=10, rot_dim=6, vdim=14, kv_rank=18, q_rank=20, window=11),
+    mamba(heads=2, vdim=9, state=33, groups=2, conv=5, norm_groups=1),
+], vocab=101, width=44, mult=0.9)
+
 # rms(difference, mean taken off) / rms(logits, mean taken off) of a row may be at most this
 TOL = {"float32": 5e-6, "bfloat16": 6e-2}
 # with the peaked scores of PEAKED, 32-bit rounding shows more (seen: 2e-5)
