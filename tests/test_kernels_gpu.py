@@ -394,11 +394,21 @@ def test_linear_fp32_few_rows(ops, M, N, K, pad):
         assert (out.cpu().double() - ref).abs().max().item() <= 3e-5
 
 
-def test_linear_bf16_refuses_odd_k(ops):
-    a = torch.zeros(4, 36, dtype=torch.bfloat16, device=DEV)
-    w = torch.zeros(8, 36, dtype=torch.bfloat16, device=DEV)
-    with pytest.raises(ops.KernelError, match="multiples of 8"):
-        ops.linear(a, w, None, torch.empty(4, 8, dtype=torch.bfloat16, device=DEV))
+@pytest.mark.parametrize("M, N, K", [(4, 8, 36), (70, 33, 44), (9, 5, 7)])
+def test_linear_bf16_takes_any_k_through_the_plain_kernel(ops, M, N, K):
+    """A K that is no multiple of 8 (the matrix-core kernels read 16 bytes at a time) runs on the plain kernel."""
+    g = torch.Generator().manual_seed(M + N + K)
+    a = _rand((M, K), torch.float32, g).to(torch.bfloat16)
+    w = _rand((N, K), torch.float32, g, std=1.0 / math.sqrt(K)).to(torch.bfloat16)
+    bias = 0.5 * _rand((N,), torch.float32, g)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), out)
+    ref = a.double() @ w.double().T + bias.double()
+    assert (out.cpu().double() - ref).abs().max().item() <= 2e-2
+    res = _rand((M, N), torch.float32, g)
+    acc = res.clone().to(DEV)
+    ops.linear(a.to(DEV), w.to(DEV), None, acc, "add_residual")
+    assert (acc.cpu().double() - (res.double() + a.double() @ w.double().T)).abs().max().item() <= 1e-4
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
