@@ -35,6 +35,8 @@ int mllm_gemm_bf16_merged(const float* split_o, const float* split_ml, int n_spl
 int mllm_ln_gemm_bf16(const float* x, int ldx, const int* rows, const float* gamma, const float* beta, float eps,
                       const void* W, int ldw, const float* bias, void* C, int ldc, int M, int N, int K, int mode,
                       hipStream_t stream);
+int mllm_rms_gemm_bf16(const float* x, int ldx, const int* rows, const float* gamma, float eps, const void* W, int ldw,
+                       const float* bias, void* C, int ldc, int M, int N, int K, int mode, hipStream_t stream);
 
 // attention.hip, attention_decode.hip, attention_prefill.hip
 int mllm_paged_attention_generic(const void* q, int q_stride, int q_col, const void* k_pages,

@@ -74,14 +74,18 @@ public:
         const int E = sh_.kv_rank + sh_.rot_dim, T = step.n_tokens, g = cache.group, H = sh_.n_heads;
         if (cache.kind != 1 || cache.k_pages.cols != E) fail("latent_attention needs pages of %d-wide rows", E);
         if (write && !own_kv_) fail("a latent-attention layer without a key/value latent of its own cannot write a cache");
-        const Tensor2& in = h.tensor(arena, s);
         Tensor2 dq = arena.tensor(F32, T, sh_.q_rank), cq = arena.tensor(dtype_, T, sh_.q_rank);
-        dq_(in, dq, STORE_F32, nullptr, s);
         const bool fill = own_kv_ && write;
         Tensor2 dkv;
-        if (fill) {
-            dkv = arena.tensor(F32, T, E);
-            dkv_(in, dkv, STORE_F32, nullptr, s);
+        if (fill) dkv = arena.tensor(F32, T, E);
+        if (T <= tuning().ln_fuse_max_rows) {
+            // few rows: each product normalises the mixer's input itself, and no norm kernel runs
+            h.linear(dq_, dq, STORE_F32, nullptr, arena, s);
+            if (fill) h.linear(dkv_, dkv, STORE_F32, nullptr, arena, s);
+        } else {
+            const Tensor2& in = h.tensor(arena, s);
+            dq_(in, dq, STORE_F32, nullptr, s);
+            if (fill) dkv_(in, dkv, STORE_F32, nullptr, s);
         }
         LatentPages pages;
         pages.rows = cache.k_pages; pages.latent_t = cache.v_pages; pages.page_size = cache.page_size;

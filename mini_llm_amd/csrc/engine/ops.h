@@ -159,6 +159,10 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
 // arrays of x's shape that lie part_stride floats apart (x the first), added in the order of their index.
 void rmsnorm(const Tensor2& x, const float* weight, float eps, int groups, const Tensor2* gate, const Tensor2& out,
              const int* rows, hipStream_t stream, int parts = 1, size_t part_stride = 0);
+// out = epilogue(rmsnorm(x[rows]) w^T + bias), the norm inside the product where the kernels allow (bfloat16, few
+// rows); `tmp` ([out.rows, K] in w's dtype) holds the normalised rows otherwise.
+void rms_linear(const Tensor2& x, const float* weight, float eps, const Tensor2& w, const float* bias, const Tensor2& out,
+                int epilogue, const int* rows, void* tmp, hipStream_t stream);
 // x += mult * scale * (y / sqrt(mean(y^2) + eps) * weight), row by row (scale: per column, or null);
 // `clear`: y is zero afterwards.
 void rmsnorm_add(const Tensor2& y, const float* weight, const float* scale, float mult, float eps, const Tensor2& x,

@@ -49,6 +49,30 @@ void rmsnorm(const Tensor2& x, const float* weight, float eps, int groups, const
           "rmsnorm");
 }
 
+void rms_linear(const Tensor2& x, const float* weight, float eps, const Tensor2& w, const float* bias, const Tensor2& out,
+                int epilogue, const int* rows, void* tmp, hipStream_t stream) {
+    need_f32(x, "rms_linear: the input");
+    need_act(w, "rms_linear: w");
+    const int64_t M = out.rows, K = x.cols;
+    if (weight == nullptr) fail("rms_linear: the norm's weight is missing");
+    if (w.cols != K || out.cols != w.rows) fail("rms_linear: rows of %lld do not fit a map of [%lld, %lld]", (long long)K, (long long)w.rows, (long long)w.cols);
+    if (rows == nullptr && x.rows != M) fail("rms_linear: out has %lld rows, the input %lld", (long long)M, (long long)x.rows);
+    const bool f32_out = epilogue == ADD_RESIDUAL || epilogue == STORE_F32;
+    if (out.dtype != (f32_out ? F32 : w.dtype)) fail("rms_linear: out must be %s", dtype_name(f32_out ? F32 : w.dtype));
+    // (more rows than that: the norm is a kernel of its own, as for the LayerNorm product)
+    if (w.dtype == BF16 && M <= tuning().ln_fuse_max_rows && K % 8 == 0 && w.stride % 8 == 0 && x.contiguous() &&
+        (reinterpret_cast<uintptr_t>(weight) & 15) == 0) {
+        const int rc = mllm_rms_gemm_bf16(static_cast<const float*>(x.data), i32(x.stride), rows, weight, eps, w.data, i32(w.stride), bias,
+                                          out.data, i32(out.stride), i32(M), i32(w.rows), i32(K), epilogue, stream);
+        if (rc == 0) return;
+        if (rc != -2) check(rc, "rms_linear");
+    }
+    if (tmp == nullptr) fail("rms_linear: these sizes need a buffer for the normalised rows");
+    Tensor2 h(tmp, w.dtype, M, K);
+    rmsnorm(x, weight, eps, 1, nullptr, h, rows, stream);
+    linear(h, w, bias, out, epilogue, nullptr, stream);
+}
+
 void rmsnorm_add(const Tensor2& y, const float* weight, const float* scale, float mult, float eps, const Tensor2& x,
                  bool clear, hipStream_t stream) {
     need_f32(y, "rmsnorm_add: y");

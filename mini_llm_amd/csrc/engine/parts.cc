@@ -559,7 +559,9 @@ StepCost DecoderModel::cost() const {
 size_t DecoderModel::workspace_bytes(int tokens, int n_logits) const {
     size_t per_layer = 0;
     for (const auto& l : layers) per_layer = std::max(per_layer, l->workspace_bytes(tokens));
-    const size_t stream = static_cast<size_t>(tokens) * hidden_size() * 4 + 256;
+    size_t stream = static_cast<size_t>(tokens) * hidden_size() * 4 + 256;
+    for (const auto& l : layers)
+        if (l->wants_zeroed_rows()) { stream *= 2; break; }
     const int rows = std::max(n_logits, 1);
     const size_t at_head = head->workspace_bytes(rows) + 2 * final_norm->workspace_bytes(rows);
     return stream + std::max(per_layer, at_head) + 4096;
@@ -574,11 +576,19 @@ void DecoderModel::forward(const StepView& step, const std::vector<CacheView>& c
     Tensor2 x = arena.tensor(F32, step.n_tokens, hidden_size());
     embedding->forward(step, position.get(), x, s);
     times.mark("embed", s);
+    StepView with_rows = step;
+    for (const auto& l : layers) {
+        if (!l->wants_zeroed_rows()) continue;
+        Tensor2 z = arena.tensor(F32, step.n_tokens, hidden_size());
+        fill_zero(z, s);
+        with_rows.zeroed_rows = static_cast<float*>(z.data);
+        break;
+    }
     for (const LayerCall& c : order) {
         if (c.cache >= static_cast<int>(caches.size()))
             fail("the execution order names cache %d, the step brings %zu caches", c.cache, caches.size());
         times.set_layer(c.layer);
-        layers[c.layer]->forward(x, step, caches[c.cache], c.write, arena, s);
+        layers[c.layer]->forward(x, with_rows, caches[c.cache], c.write, arena, s);
     }
     times.set_layer(-1);
     if (step.n_logits == 0) { times.end_step(s); return; }

@@ -93,6 +93,8 @@ struct StepView {
     const int* starts = nullptr;       // [B]
     const int* state_slots = nullptr;  // [B]
     const int* logit_rows = nullptr;   // [n_logits]
+    float* zeroed_rows = nullptr;      // fp32 [n_tokens, hidden], all zero, if a layer asked for it (Block::wants_zeroed_rows):
+                                       // room for a sub-layer's result; whoever uses it leaves it zero again
     int n_groups = 0;
     const int* const* block_tables = nullptr;   // per group [B, max_blocks[g]]
     const int* max_blocks = nullptr;            // per group
@@ -253,6 +255,9 @@ public:
                          hipStream_t s) const = 0;
     virtual size_t workspace_bytes(int tokens) const = 0;
     virtual CacheNeed cache_need() const = 0;             // its mixer's
+    // true: the model keeps one cleared fp32 buffer of the stream's shape for the step (StepView::zeroed_rows),
+    // cleared once, instead of every layer clearing one of its own
+    virtual bool wants_zeroed_rows() const { return false; }
     virtual void reserve(int max_seqs, hipStream_t s) const = 0;
     virtual void add_cost(StepCost&) const = 0;
 };

@@ -28,6 +28,15 @@ public:
         rmsnorm(x, weight_, eps_, 1, nullptr, h, rows, s);
         return h;
     }
+    void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,
+                const KvScatter* kv, Arena& arena, hipStream_t s) const override {
+        if (kv != nullptr) { Norm::linear(x, lin, out, epilogue, rows, kv, arena, s); return; }
+        // the norm inside the product where the kernels allow it; otherwise the rows pass through the arena
+        const size_t mark = arena.mark();
+        void* tmp = arena.take(static_cast<size_t>(out.rows) * size_ * dtype_size(lin.weight.dtype));
+        rms_linear(x, weight_, eps_, lin.weight, lin.bias, out, epilogue, rows, tmp, s);
+        arena.release(mark);
+    }
     void add_scaled(const Tensor2& y, const float* scale, float mult, const Tensor2& x, bool clear, hipStream_t s) const override {
         if (y.cols != size_) fail("rmsnorm: rows of %lld, the norm is %d wide", (long long)y.cols, size_);
         rmsnorm_add(y, weight_, scale, mult, eps_, x, clear, s);
@@ -65,8 +74,11 @@ public:
     void forward(const Tensor2& x, const StepView& step, const CacheView& cache, bool write, Arena& arena,
                  hipStream_t s) const override {
         const size_t outer = arena.mark();
-        Tensor2 y = arena.tensor(F32, x.rows, x.cols);
-        fill_zero(y, s);
+        // the sub-layer's result: the step's cleared buffer (left cleared again by the norms behind the
+        // sub-layers), or one of this layer's own
+        const bool shared = step.zeroed_rows != nullptr;
+        Tensor2 y = shared ? Tensor2(step.zeroed_rows, F32, x.rows, x.cols) : arena.tensor(F32, x.rows, x.cols);
+        if (!shared) fill_zero(y, s);
         const size_t mark = arena.mark();
         {
             NormedInput h(*pre1_, x);
@@ -74,7 +86,7 @@ public:
         }
         arena.release(mark);
         if (x.cols != size_) fail("a sandwich-norm block of width %d was handed a stream of %lld", size_, (long long)x.cols);
-        post1_->add_scaled(y, static_cast<const float*>(scale1_.data), mult_, x, ff_ != nullptr, s);
+        post1_->add_scaled(y, static_cast<const float*>(scale1_.data), mult_, x, shared || ff_ != nullptr, s);
         StageTimes::get().mark("post_norm", s);
         if (ff_) {
             {
@@ -82,7 +94,7 @@ public:
                 ff_->forward(h, step, y, arena, s);
             }
             arena.release(mark);
-            post2_->add_scaled(y, static_cast<const float*>(scale2_.data), mult_, x, false, s);
+            post2_->add_scaled(y, static_cast<const float*>(scale2_.data), mult_, x, shared, s);
             StageTimes::get().mark("post_norm2", s);
         }
         arena.release(outer);
@@ -93,6 +105,7 @@ public:
         return a + static_cast<size_t>(tokens) * size_ * 4 + 1024;
     }
     CacheNeed cache_need() const override { return mixer_->cache_need(); }
+    bool wants_zeroed_rows() const override { return true; }
     void reserve(int max_seqs, hipStream_t s) const override {
         mixer_->reserve(max_seqs, s);
         if (ff_) ff_->reserve(max_seqs, s);
@@ -136,10 +149,16 @@ public:
     }
     void forward(NormedInput& h, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s) const override {
         const int T = step.n_tokens, F = up_.out_features();
-        const Tensor2& in = h.tensor(arena, s);
         Tensor2 g = arena.tensor(dtype_, T, F), u = arena.tensor(dtype_, T, F);
-        gate_(in, g, STORE, nullptr, s);
-        up_(in, u, STORE, nullptr, s);
+        if (T <= tuning().ln_fuse_max_rows) {
+            // few rows: each product normalises its input itself, and no norm kernel runs
+            h.linear(gate_, g, STORE, nullptr, arena, s);
+            h.linear(up_, u, STORE, nullptr, arena, s);
+        } else {
+            const Tensor2& in = h.tensor(arena, s);
+            gate_(in, g, STORE, nullptr, s);
+            up_(in, u, STORE, nullptr, s);
+        }
         StageTimes::get().mark("fc1", s);
         glu_clamped(g, u, limit_, alpha_, g, s);            // in place over the gate's rows
         down_(g, x, ADD_RESIDUAL, nullptr, s);

@@ -415,7 +415,9 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
                  // A_MERGED: the attention splits' states (layout: attention_decode.hip), their number,
                  // heads per token and head size (K = heads x head size)
                  const float* __restrict__ split_o = nullptr, const float* __restrict__ split_ml = nullptr,
-                 int n_splits = 1, int a_heads = 1, int a_head_dim = 8) {
+                 int n_splits = 1, int a_heads = 1, int a_head_dim = 8,
+                 // A_NORMED: != 0: the norm does not centre (RMS norm: x / sqrt(mean(x^2) + eps) * gamma)
+                 int rms = 0) {
     // NT > 1 (SPLIT_K, MT == 1): the workgroup owns cols_per_wg <= 16 NT columns, NT tiles that share
     // the rows of A, the last one possibly narrower: for products with more than 256 tiles, whose
     // columns are dealt out evenly to 256 workgroups (one per compute unit; a kernel of this size
@@ -798,7 +800,7 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
 #pragma unroll
             for (int u = 0; u < 8; ++u)
                 if (u < n_u && lane + 64 * u < nq) sum += (v[j][u].x + v[j][u].y) + (v[j][u].z + v[j][u].w);
-            mean[j] = wave_sum(sum) / static_cast<float>(K);
+            mean[j] = rms ? 0.f : wave_sum(sum) / static_cast<float>(K);
             float q = 0.f;
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
@@ -949,7 +951,7 @@ template <bool LN_FUSED, bool MERGED = false>
 static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const float* bias, void* C, int ldc,
                          int M, int N, int K, int mode, const float* gamma, const float* beta, float eps,
                          const int* rows, hipStream_t stream, void* workspace = nullptr, size_t workspace_bytes = 0,
-                         MergedA merged = MergedA{}) {
+                         MergedA merged = MergedA{}, int rms = 0) {
     static_assert(!(LN_FUSED && MERGED), "one source of A");
     const int tiles = (N + 15) / 16;
     const bool split_k = tiles < 1024;
@@ -1034,7 +1036,7 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
         if (e != hipSuccess) return static_cast<int>(e);                                               \
         kernel<<<grid, block, staged_bytes, stream>>>(W, ldw, N, K, M, col_blocks, row_blocks, 16, 1, A, lda, mode, \
                                                       bias, C, ldc, gamma, beta, eps, rows, nullptr, nullptr, \
-                                                      nullptr, nullptr, 1, 1, 8);                      \
+                                                      nullptr, nullptr, 1, 1, 8, 0);                   \
         break;                                                                                         \
     }
         switch (mt) {
@@ -1065,7 +1067,7 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
         kernel<<<grid, block, smem, stream>>>(W, ldw, N, K, M, col_blocks, row_blocks, cols_per_wg, k_parts, A, lda, \
                                               mode, bias, C, ldc, gamma, beta, eps, rows, part_sums,      \
                                               part_counters, merged.split_o, merged.split_ml, merged.n_splits, \
-                                              merged.heads, merged.head_dim);                          \
+                                              merged.heads, merged.head_dim, rms);                     \
     } while (0)
     if (split_k) {
         // a chunk holds all k blocks of a wavefront when they are at most 3 (4 without the fused
@@ -1256,6 +1258,19 @@ int mllm_ln_gemm_bf16(const float* x, int ldx, const int* rows, const float* gam
     if (M > 64) return -2;
     int rc = launch_skinny<true>(x, ldx, static_cast<const bf16_t*>(W), ldw, bias, C, ldc, M, N, K, mode, gamma,
                                  beta, eps, rows, stream);
+    if (rc != 0) return rc;
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+// The same with an RMS norm in front of the product: C = epilogue((x / sqrt(mean(x^2) + eps) * gamma) W^T + bias).
+int mllm_rms_gemm_bf16(const float* x, int ldx, const int* rows, const float* gamma, float eps, const void* W, int ldw,
+                       const float* bias, void* C, int ldc, int M, int N, int K, int mode, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K % 8 != 0 || ldw % 8 != 0 || (reinterpret_cast<uintptr_t>(W) & 15)) return -1;
+    if (M > 64) return -2;
+    int rc = launch_skinny<true>(x, ldx, static_cast<const bf16_t*>(W), ldw, bias, C, ldc, M, N, K, mode, gamma,
+                                 nullptr, eps, rows, stream, nullptr, 0, MergedA{}, 1);
     if (rc != 0) return rc;
     MLLM_LAUNCH_CHECK();
     return 0;

@@ -295,11 +295,12 @@ def test_toy_architecture_through_the_benchmark(tmp_path):
     rec = json.loads(r.stdout.strip().splitlines()[-1])
     assert rec["config"]["model"] == "ToyLM-sizes" and rec["config"]["vocab_size"] == 203 and rec["value"] > 0
     # weights a step reads: the attention layer's, the stateful layer's, the final norm's and the tied head's (bf16
-    # matrices, fp32 vectors); the cache: one layer of one key/value head of 16
+    # matrices, fp32 vectors); the cache: one layer of one key/value head of 16; the stateful layer's state of every
+    # request (D floats), read and written once a step
     D, dh = 48, 16
     matrices = (D + 2 * dh) * D + D * D + 2 * D * D * 2 + 203 * D
     vectors = 2 * D + D + 2 * D + D + 2 * D
-    live = 4 * rec["config"]["mean_context"] * 2 * dh * 2
+    live = 4 * rec["config"]["mean_context"] * 2 * dh * 2 + 4 * 2 * D * 4
     assert rec["roofline"]["bytes_per_step"] == int(2 * matrices + 4 * vectors + live)
 
 
