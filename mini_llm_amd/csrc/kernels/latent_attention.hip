@@ -32,26 +32,53 @@ latent_prepare_kernel(const float* __restrict__ dq, int ld_dq, int Rq, const flo
                       T* __restrict__ pages, T* __restrict__ vt_pages, int page_size, const int* __restrict__ slots,
                       const int* __restrict__ positions, float eps, double log2_base, int rot_dims) {
     const int t = blockIdx.x, lane = threadIdx.x;
+    // Up to 8 values a lane of each latent are requested up front, without conditions (a loop of unknown length
+    // would wait for every load before it asks for the next); longer latents read the rest in a loop.
+    const float* qrow = dq + static_cast<size_t>(t) * ld_dq;
+    const int slot = dkv ? slots[t] : -1;
+    const bool fill = dkv != nullptr && slot >= 0;
+    const float* row = fill ? dkv + static_cast<size_t>(t) * ld_dkv : qrow;
+    const int Rk = fill ? R : Rq;                              // (no latent to fill: the loads below repeat the query's)
+    float qv[8], kv[8], qw[8], kw[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int iq = min(lane + 64 * u, Rq - 1), ik = min(lane + 64 * u, Rk - 1);
+        qv[u] = qrow[iq];
+        qw[u] = wq[iq];
+        kv[u] = row[ik];
+        kw[u] = fill ? wkv[ik] : 0.f;
+    }
     {
-        const float* row = dq + static_cast<size_t>(t) * ld_dq;
         float ss = 0.f;
-        for (int i = lane; i < Rq; i += 64) ss += row[i] * row[i];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) if (lane + 64 * u < Rq) ss += qv[u] * qv[u];
+        for (int i = lane + 512; i < Rq; i += 64) ss += qrow[i] * qrow[i];
         const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(Rq) + eps);
         T* o = cq + static_cast<size_t>(t) * ld_cq;
-        for (int i = lane; i < Rq; i += 64) o[i] = from_float<T>(row[i] * inv * wq[i]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) if (lane + 64 * u < Rq) o[lane + 64 * u] = from_float<T>(qv[u] * inv * qw[u]);
+        for (int i = lane + 512; i < Rq; i += 64) o[i] = from_float<T>(qrow[i] * inv * wq[i]);
     }
-    if (dkv == nullptr) return;
-    const int slot = slots[t];
-    if (slot < 0) return;
-    const float* row = dkv + static_cast<size_t>(t) * ld_dkv;
+    if (!fill) return;
     T* o = pages + static_cast<size_t>(slot) * (R + Dr);
     float ss = 0.f;
-    for (int i = lane; i < R; i += 64) ss += row[i] * row[i];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) if (lane + 64 * u < R) ss += kv[u] * kv[u];
+    for (int i = lane + 512; i < R; i += 64) ss += row[i] * row[i];
     const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(R) + eps);
     // (vt_pages, optional: the latent once more, transposed page by page, [page][R][page_size], which is the
     // operand shape of the matrix-core kernel's second product)
     T* vt = vt_pages ? vt_pages + static_cast<size_t>(slot / page_size) * page_size * R + slot % page_size : nullptr;
-    for (int i = lane; i < R; i += 64) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int i = lane + 64 * u;
+        if (i < R) {
+            const T c = from_float<T>(kv[u] * inv * kw[u]);
+            o[i] = c;
+            if (vt) vt[static_cast<size_t>(i) * page_size] = c;
+        }
+    }
+    for (int i = lane + 512; i < R; i += 64) {
         const T c = from_float<T>(row[i] * inv * wkv[i]);
         o[i] = c;
         if (vt) vt[static_cast<size_t>(i) * page_size] = c;

@@ -104,7 +104,7 @@ rmsnorm_add_kernel(float* __restrict__ y, const float* __restrict__ w, const flo
 // first use (a load under a condition waits for all loads in flight, and a row of 768 then costs eight round trips).
 // `parts` > 1: the input is the sum of that many arrays `part_stride` floats apart (partial results of a kernel
 // that splits a sum over workgroups), added in the order of their index.
-template <typename OutT, int WAVES>
+template <typename OutT, int WAVES, bool SHARES = false>
 __global__ void __launch_bounds__(64 * WAVES)
 rmsnorm_vec_kernel(const float* __restrict__ x, int ldx, const int* __restrict__ rows, const float* __restrict__ w,
                    const float* __restrict__ gate, int ldg, OutT* __restrict__ y, int ldy, int n, int D, int groups,
@@ -122,14 +122,24 @@ rmsnorm_vec_kernel(const float* __restrict__ x, int ldx, const int* __restrict__
 #pragma unroll
     for (int u = 0; u < 8; ++u)
         if (u < n_u) v[u] = xr[min(lane + 64 * u, nq - 1)];
-    for (int part = 1; part < parts; ++part) {
-        const float4* xp = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(xr) + part * part_stride);
+    if (SHARES) {
+        // up to four shares (the launcher sends more to the plain kernel): all of them requested before the first
+        // is added, a share beyond `parts` read from the last one and not added
+        float4 sh[3][8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
-            if (u < n_u) {
-                const float4 a = xp[min(lane + 64 * u, nq - 1)];
-                v[u].x += a.x; v[u].y += a.y; v[u].z += a.z; v[u].w += a.w;
-            }
+        for (int part = 1; part < 4; ++part) {
+            const float4* xp = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(xr) + min(part, parts - 1) * part_stride);
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (u < n_u) sh[part - 1][u] = xp[min(lane + 64 * u, nq - 1)];
+        }
+#pragma unroll
+        for (int part = 1; part < 4; ++part)
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (u < n_u && part < parts) {
+                    v[u].x += sh[part - 1][u].x; v[u].y += sh[part - 1][u].y; v[u].z += sh[part - 1][u].z; v[u].w += sh[part - 1][u].w;
+                }
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u)
@@ -240,7 +250,7 @@ int mllm_rmsnorm(const float* x, int ldx, const int* rows, const float* w, const
     if (groups < 1 || D % groups != 0 || parts < 1) return -1;
     const long long pairs = static_cast<long long>(n) * groups;
     const int Dg = D / groups, esz = out_dtype == MLLM_F32 ? 4 : 2;
-    const bool vec = Dg % 4 == 0 && Dg <= 2048 && ldx % 4 == 0 && (gate == nullptr || ldg % 4 == 0) && part_stride % 4 == 0 &&
+    const bool vec = parts <= 4 && Dg % 4 == 0 && Dg <= 2048 && ldx % 4 == 0 && (gate == nullptr || ldg % 4 == 0) && part_stride % 4 == 0 &&
                      (static_cast<size_t>(ldy) * esz) % 16 == 0 && (static_cast<size_t>(Dg) * esz) % 8 == 0 &&
                      ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(gate) |
                        reinterpret_cast<uintptr_t>(y)) & 15) == 0;
@@ -248,13 +258,19 @@ int mllm_rmsnorm(const float* x, int ldx, const int* rows, const float* w, const
 #define RMS(KERNEL, TYPE, WAVES)                                                                                        \
     KERNEL<TYPE, WAVES><<<static_cast<int>((pairs + WAVES - 1) / WAVES), 64 * WAVES, 0, stream>>>(                      \
         x, ldx, rows, w, gate, ldg, static_cast<TYPE*>(y), ldy, n, D, groups, eps, parts, part_stride)
-    if (vec) {
+#define RMS_SHARES(TYPE)                                                                                                \
+    rmsnorm_vec_kernel<TYPE, 4, true><<<static_cast<int>((pairs + 3) / 4), 256, 0, stream>>>(                           \
+        x, ldx, rows, w, gate, ldg, static_cast<TYPE*>(y), ldy, n, D, groups, eps, parts, part_stride)
+    if (vec && parts > 1) {
+        if (out_dtype == MLLM_F32) RMS_SHARES(float); else RMS_SHARES(bf16_t);
+    } else if (vec) {
         if (out_dtype == MLLM_F32) { if (pairs >= 512) RMS(rmsnorm_vec_kernel, float, 8); else RMS(rmsnorm_vec_kernel, float, 4); }
         else { if (pairs >= 512) RMS(rmsnorm_vec_kernel, bf16_t, 8); else RMS(rmsnorm_vec_kernel, bf16_t, 4); }
     } else {
         if (out_dtype == MLLM_F32) RMS(rmsnorm_kernel, float, 4); else RMS(rmsnorm_kernel, bf16_t, 4);
     }
 #undef RMS
+#undef RMS_SHARES
     MLLM_LAUNCH_CHECK();
     return 0;
 }

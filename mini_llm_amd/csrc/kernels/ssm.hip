@@ -19,21 +19,24 @@ __device__ __forceinline__ float softplus_precise(float v) { return fmaxf(v, 0.f
 __global__ void conv_silu_kernel(const float* __restrict__ proj, int ld, int col0, int C, const float* __restrict__ w,
                                  const float* __restrict__ bias, int taps, const int* __restrict__ token_seq,
                                  const int* __restrict__ cu_q, const int* __restrict__ state_slots,
-                                 const float* __restrict__ state, size_t slot_floats, float* __restrict__ out, int ldo,
-                                 long long total) {
+                                 float* __restrict__ state, size_t slot_floats, float* __restrict__ out, int ldo,
+                                 long long total, int carry) {
     const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const int t = static_cast<int>(i / C), ch = static_cast<int>(i % C);
     const int b = token_seq[t], slot = state_slots[b];
     if (slot < 0) return;
     const int first = cu_q[b], k = t - first;
-    const float* carried = state + static_cast<size_t>(slot) * slot_floats;
+    float* carried = state + static_cast<size_t>(slot) * slot_floats;
     float acc = bias[ch];
     for (int j = 0; j < taps; ++j) {
         const int idx = k - (taps - 1 - j);
         const float v = idx >= 0 ? proj[static_cast<size_t>(first + idx) * ld + col0 + ch]
                                  : carried[static_cast<size_t>(taps - 1 + idx) * C + ch];
         acc += w[static_cast<size_t>(ch) * taps + j] * v;
+        // `carry` (every portion of the step is a single token, so this thread is the channel's only reader): the
+        // carried rows move up by one behind the read, and the token's input becomes the newest
+        if (carry && j >= 1) carried[static_cast<size_t>(j - 1) * C + ch] = v;
     }
     out[static_cast<size_t>(t) * ldo + ch] = silu_precise(acc);
 }
@@ -389,10 +392,12 @@ int mllm_conv_silu(const float* proj, int ld, int col0, int C, const float* w, c
     if (T <= 0 || C <= 0) return 0;
     if (taps < 1 || taps > 16) return -1;
     const long long total = static_cast<long long>(T) * C;
+    // (one token a sequence: the convolution's kernel brings the carried rows up to date itself)
+    const bool single = T == B && write && taps > 1;
     conv_silu_kernel<<<static_cast<int>((total + 255) / 256), 256, 0, stream>>>(proj, ld, col0, C, w, bias, taps, token_seq, cu_q,
-                                                                                state_slots, state, slot_floats, out, ldo, total);
+                                                                                state_slots, state, slot_floats, out, ldo, total, single ? 1 : 0);
     MLLM_LAUNCH_CHECK();
-    if (write && taps > 1) {
+    if (write && taps > 1 && !single) {
         const long long pairs = static_cast<long long>(B) * C;
         conv_carry_kernel<<<static_cast<int>((pairs + 255) / 256), 256, 0, stream>>>(proj, ld, col0, C, taps, cu_q, state_slots, state,
                                                                                     slot_floats, B);
