@@ -35,12 +35,12 @@ def small_config(n_layer, size="gpt2-small", n_positions=1024):
 def kugulorn_config(n_layer, size="gpt2-small", n_positions=1024):
     """A Kugulorn model of about the size of the GPT-2 configuration `size`: the same width, number of layers,
     vocabulary and context; Mamba-2 layers (inner width twice the model's, heads of 64, a state of 128 rows) and
-    latent-attention layers (as many heads as GPT-2 has, a latent of a third of the width beside 32 rotated
+    latent-attention layers (as many heads as GPT-2 has, a latent of up to a third of the width beside 32 rotated
     columns, every second one reading the pages of the one before it, the window as long as the context) in
     turn, each with a gated feed-forward whose three matrices hold what GPT-2's two do."""
     full_layers, d, h, f = SIZES[size]
     n = n_layer or full_layers
-    rank = max(64, d // 3 // 32 * 32)                    # 256 at 768, 320 at 1024, 512 at 1600
+    rank = max(r for r in (64, 128, 256, 512) if r <= max(64, d // 3))      # 256 at 768 and 1,024, 512 at 1,600
     ff = f * 2 // 3 // 64 * 64
     mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
     layers, last_own = [], None

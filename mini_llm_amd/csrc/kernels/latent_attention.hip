@@ -338,8 +338,10 @@ latent_expand_kernel(const T* __restrict__ o_lat, int ldo, const T* __restrict__
 // The second product's A operand needs 8 keys of one latent column side by side, which the page-transposed
 // copy of the latent holds ([page][R][page_size]): its 16-byte pieces go to LDS as they are, keys outside
 // the tile's range set to zero (a page's tail may hold anything). E = 32 * KS, R = 16 * DT.
+// (The widest sizes keep 128 accumulators, 70 query registers and a tile's staging registers a lane: they get the
+// whole register file, one wavefront per SIMD, which is also all their LDS allows.)
 template <int KS, int DT>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2)))
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, (KS + DT > 30) ? 1 : 2)))
 latent_prefill_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
                       const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
                       const int* __restrict__ ctx_len, int n_seqs, int H, int page_size, float scale_log2e, int window,
@@ -661,7 +663,7 @@ int mllm_latent_attention(const void* qa, int ldqa, const void* pages, const int
 // nsplit > 1: every row's key tiles are shared by nsplit workgroups whose states meet in `partials`
 // (n_rows * nsplit * (R + 2) floats, n_rows = T*H) and are merged by a second kernel. single_tokens != 0: every
 // sequence brings exactly one token (n_tiles_upper is then n_seqs * ceil(H / 64)). n_tiles_upper: an upper bound of sum over sequences of ceil(q_len * H / 64). Returns -2 when the
-// sizes are not ones it is built for (E and R among (128, 96), (96, 64), (160, 128), (288, 256), (576, 512);
+// sizes are not ones it is built for (E and R among (128, 96), (96, 64), (160, 128), (288, 256), (544, 512), (576, 512);
 // page sizes 8 to 64, powers of two; a block table that fits the LDS beside the tiles): the caller then runs
 // mllm_latent_attention.
 int mllm_latent_attention_tiles(const void* qa, const void* k_pages, const void* vt_pages, const int* block_tables,
@@ -699,7 +701,7 @@ int mllm_latent_attention_tiles(const void* qa, const void* k_pages, const void*
         }                                                                                                            \
         return 0;                                                                                                    \
     }
-    LP_CASE(4, 6) LP_CASE(3, 4) LP_CASE(5, 8) LP_CASE(9, 16) LP_CASE(18, 32)
+    LP_CASE(4, 6) LP_CASE(3, 4) LP_CASE(5, 8) LP_CASE(9, 16) LP_CASE(17, 32) LP_CASE(18, 32)
 #undef LP_CASE
     return -2;
 }

@@ -66,6 +66,12 @@ TILED = model([
     latent(heads=2, dim=24, rot_dim=32, vdim=8, kv_rank=128, q_rank=16, window=70, kv_from=2),
 ], vocab=211, width=56, mult=0.6)
 
+# the widest cached rows of the matrix-core kernel: latents of 512 beside 32 and 64 rotated columns
+WIDE = model([
+    latent(heads=2, dim=16, rot_dim=32, vdim=8, kv_rank=512, q_rank=16, window=90),
+    latent(heads=3, dim=8, rot_dim=64, vdim=8, kv_rank=512, q_rank=8, window=200),
+], vocab=97, width=32, mult=0.5)
+
 # sizes that are multiples of neither 8 nor 4: the plain bfloat16 product, the scan without staging, rows of the
 # pages that are not 16-byte pieces
 ODD = model([

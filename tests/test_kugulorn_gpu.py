@@ -87,6 +87,18 @@ def test_prompt_portions_on_the_matrix_cores(dirs, family, page):
     assert runner.check() == "" and runner.info()["n_requests"] == 0
 
 
+@pytest.mark.parametrize("family", ["whole", "mixed"])
+def test_widest_rows_on_the_matrix_cores(dirs, family):
+    from mini_llm_amd.kernels import ops
+    cfg, d = kc.WIDE, dirs("WIDE")
+    reqs = kc.requests(cfg["vocab"], [3, 70, 129, 260], seed=73)
+    steps = _families(reqs, seed=7)[family]
+    ops.reset_seen()
+    runner = _runner(d, "bfloat16", n_pages=ru.peak_tokens(steps) // 16, page=16)
+    kc.check_against_plain(d, reqs, steps, ru.run_in_process(runner, steps), "bfloat16", cfg["vocab"], f"wide {family}")
+    assert ops.seen("latent_tile_launches") > 0 and ops.seen("latent_token_launches") == 0
+
+
 def test_matrix_core_kernel_against_the_per_token_kernel(dirs):
     """The same whole prompts with the matrix-core kernel switched off: both kernels round differently, no more."""
     from mini_llm_amd.kernels import ops
