@@ -56,6 +56,9 @@ MIXED_B = model([
 # scores that one key dominates: a window that is one key off, or a key lost at a page's border, changes a row
 PEAKED = model([latent(window=5, scale=6.0), latent(window=16, scale=6.0, heads=1), latent(window=6, scale=6.0, kv_from=1)], width=32)
 
+# the same with windows of hundreds of keys: a single far key often carries a row
+PEAKED_FAR = model([latent(window=300, scale=5.0), latent(window=190, scale=5.0, heads=3, kv_from=0)], width=32)
+
 # cached rows of 96 and 160 columns (latents of 64 and 128): sizes that the matrix-core kernel of prompt portions
 # takes at pages of 16 tokens in bfloat16; windows shorter and longer than its 64-key tiles; 3 and 5 heads, so
 # that a tile of 64 (token, head) rows starts and ends in the middle of a token

@@ -133,6 +133,19 @@ def test_window_and_page_borders_with_peaked_scores(dirs, page):
                                tol=kc.TOL_PEAKED)
 
 
+@pytest.mark.parametrize("page", [4, 16])
+def test_far_keys_among_hundreds_with_peaked_scores(dirs, page):
+    """Windows of 300 and 190 keys and scores that single keys dominate: a key far back that is lost (a page of the
+    table, a tile's edge, a window that ends early) changes whole rows. Prompts, portions and decoding, 32-bit."""
+    cfg, d = kc.PEAKED_FAR, dirs("PEAKED_FAR")
+    reqs = kc.requests(cfg["vocab"], [330, 200], seed=23)
+    for label, steps in (("whole", ru.trace_whole(reqs)), ("decode", ru.trace_decode_tail(reqs, tail=40)),
+                         ("chunks", ru.trace_chunks(reqs, seed=4, sizes=(2, 70, 3, 129, 16)))):
+        runner = _runner(d, "float32", n_pages=-(-ru.peak_tokens(steps) // page), page=page)
+        kc.check_against_plain(d, reqs, steps, ru.run_in_process(runner, steps), "float32", cfg["vocab"], f"far keys page {page} {label}",
+                               tol=kc.TOL_PEAKED)
+
+
 def test_peaked_scores_would_show_a_window_one_key_off(dirs):
     """The test above has teeth: the plain model with every window one key wider differs from the plain model
     by far more than the tolerance, in most rows."""
