@@ -47,7 +47,6 @@ public:
             fail("latent_attention: heads and sizes must be positive");
         if (sh_.rot_dim % 2 != 0 || sh_.rot_dims % 2 != 0 || sh_.rot_dims > sh_.rot_dim || sh_.rot_dims < 0)
             fail("latent_attention: %d of %d rotated columns: both must be even, the first at most the second", sh_.rot_dims, sh_.rot_dim);
-        if (dtype_ == BF16 && (sh_.kv_rank + sh_.rot_dim) % 2 != 0) fail("latent_attention: a cached row of %d bfloat16 columns is not supported", sh_.kv_rank + sh_.rot_dim);
         const int qd = sh_.n_heads * (sh_.plain_dim + sh_.rot_dim);
         dq_ = Linear(p.weights("dq.weight"), nullptr);
         uq_ = Linear(p.weights("uq.weight"), nullptr);

@@ -213,7 +213,6 @@ void latent_attention(const Tensor2& qa, const LatentPages& pages, const LatentS
         fail("latent_attention: the result must be [T, %d]", sh.n_heads * sh.kv_rank);
     if (step.block_tables == nullptr || step.token_seq == nullptr || step.positions == nullptr || step.max_blocks < 1)
         fail("latent_attention: block tables, token_seq and positions are needed");
-    if (qa.dtype == BF16 && E % 2 != 0) fail("latent_attention: rows of %d bfloat16 columns are not supported (an even number is)", E);
     if (window < 0) fail("latent_attention: a negative window");
     // the matrix-core kernel: one workgroup per 64 (token, head) rows of a sequence
     if (tuning().latent_tiles && qa.dtype == BF16 && pages.latent_t.data != nullptr && step.cu_q != nullptr &&

@@ -229,30 +229,43 @@ latent_attention_kernel(const T* __restrict__ qa, int ldqa, const T* __restrict_
                         int R, int Dr, int page_size, float scale_log2, int window, T* __restrict__ o_lat, int ldo, int KS) {
     extern __shared__ float lds[];
     const int E = R + Dr;
+    // (bfloat16 rows are read two columns a word: an odd row gets one more column, zero in the queries and in LDS)
+    const int Eq = sizeof(T) == 2 ? E + (E & 1) : E;
     float* q_s = lds;
-    float* o_s = q_s + HG * E;
+    float* o_s = q_s + HG * Eq;
     float* p_s = o_s + HG * R;
     T* k_s = reinterpret_cast<T*>(p_s + 4 * 64);
     const int t = blockIdx.x, h0 = blockIdx.y * HG, nh = min(HG, H - h0);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
     const int pos = positions[t];
     const int* table = block_tables + static_cast<size_t>(token_seq[t]) * max_blocks;
-    for (int i = threadIdx.x; i < nh * E; i += 256)
-        q_s[i] = to_float(qa[static_cast<size_t>(t) * ldqa + h0 * E + i]) * scale_log2;
+    for (int i = threadIdx.x; i < nh * Eq; i += 256) {
+        const int hh = i / Eq, c = i % Eq;
+        q_s[i] = c < E ? to_float(qa[static_cast<size_t>(t) * ldqa + (h0 + hh) * E + c]) * scale_log2 : 0.f;
+    }
     for (int i = threadIdx.x; i < nh * R; i += 256) o_s[i] = 0.f;
     // per head of this wavefront: running maximum and sum (up to 8 heads a wavefront: HG <= 32)
     float m_run[8], l_run[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u) { m_run[u] = -INFINITY; l_run[u] = 0.f; }
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int words = sizeof(T) == 2 ? E / 2 : E;           // 32-bit words of a key row (E even for bfloat16)
+    const int words = sizeof(T) == 2 ? Eq / 2 : E;          // 32-bit words of a key row in LDS
+    const bool by_words = sizeof(T) == 4 || (E & 1) == 0;   // (an odd bfloat16 row does not start on a word)
     for (int k0 = lo; k0 <= pos; k0 += 64) {
         const int nk = min(64, pos + 1 - k0);
         __syncthreads();                                   // the tile before is used up
-        for (int i = threadIdx.x; i < nk * words; i += 256) {
-            const int j = i / words, c = i % words, kp = k0 + j;
-            const size_t row = static_cast<size_t>(table[kp / page_size]) * page_size + kp % page_size;
-            reinterpret_cast<uint32_t*>(k_s)[j * KS + c] = reinterpret_cast<const uint32_t*>(pages + row * E)[c];
+        if (by_words) {
+            for (int i = threadIdx.x; i < nk * words; i += 256) {
+                const int j = i / words, c = i % words, kp = k0 + j;
+                const size_t row = static_cast<size_t>(table[kp / page_size]) * page_size + kp % page_size;
+                reinterpret_cast<uint32_t*>(k_s)[j * KS + c] = reinterpret_cast<const uint32_t*>(pages + row * E)[c];
+            }
+        } else {
+            for (int i = threadIdx.x; i < nk * Eq; i += 256) {
+                const int j = i / Eq, c = i % Eq, kp = k0 + j;
+                const size_t row = static_cast<size_t>(table[kp / page_size]) * page_size + kp % page_size;
+                k_s[static_cast<size_t>(j) * 2 * KS + c] = c < E ? pages[row * E + c] : from_float<T>(0.f);
+            }
         }
         __syncthreads();
         const uint32_t* kw = reinterpret_cast<const uint32_t*>(k_s) + min(lane, nk - 1) * KS;
@@ -260,7 +273,7 @@ latent_attention_kernel(const T* __restrict__ qa, int ldqa, const T* __restrict_
         for (int u = 0; u < 8; ++u) {
             const int hh = wave + 4 * u;
             if (hh < nh) {
-                const float* qh = q_s + hh * E;
+                const float* qh = q_s + hh * Eq;
                 float s = 0.f;
                 if (sizeof(T) == 2) {
                     for (int c = 0; c < words; ++c) {
@@ -619,19 +632,19 @@ int mllm_latent_absorb(const void* q, int ldq, const void* w_uk, int ldw, void* 
     return 0;
 }
 
-// See latent_attention_kernel. -1: sizes the kernel's accesses do not allow (E odd in bfloat16); -2: a head's
-// rows do not fit the LDS.
+// See latent_attention_kernel. -1: sizes the kernel's accesses do not allow; -2: a head's rows do not fit the LDS.
 int mllm_latent_attention(const void* qa, int ldqa, const void* pages, const int* block_tables, int max_blocks,
                           const int* token_seq, const int* positions, int T, int H, int R, int Dr, int page_size, float scale,
                           int window, void* o_lat, int ldo, int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
     const int E = R + Dr, esz = dtype == MLLM_F32 ? 4 : 2;
-    if (H < 1 || R < 1 || Dr < 0 || page_size < 1 || (dtype != MLLM_F32 && E % 2 != 0)) return -1;
+    if (H < 1 || R < 1 || Dr < 0 || page_size < 1) return -1;
     if ((reinterpret_cast<uintptr_t>(pages) & 3) != 0) return -1;
-    int words = dtype == MLLM_F32 ? E : E / 2;
+    const int Eq = dtype == MLLM_F32 ? E : E + (E & 1);
+    int words = dtype == MLLM_F32 ? E : Eq / 2;
     const int KS = words | 1;                                    // an odd row stride, in 32-bit words
     auto lds_for = [&](int hg) {
-        return static_cast<size_t>(hg) * (E + R) * 4 + 4 * 64 * 4 + static_cast<size_t>(64) * KS * 4;
+        return static_cast<size_t>(hg) * (Eq + R) * 4 + 4 * 64 * 4 + static_cast<size_t>(64) * KS * 4;
     };
     int HG = std::min(H, 32);
     while (HG > 1 && lds_for(HG) > static_cast<size_t>(MAX_LDS)) HG = (HG + 1) / 2;

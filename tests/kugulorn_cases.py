@@ -81,6 +81,7 @@ ODD = model([
     mamba(heads=3, vdim=12, state=10, groups=1, conv=2, norm_groups=3, mlp=dense(52, 1.0)),
     latent(heads=3, dim=10, rot_dim=6, vdim=14, kv_rank=18, q_rank=20, window=11),
     mamba(heads=2, vdim=9, state=33, groups=2, conv=5, norm_groups=1),
+    latent(heads=2, dim=7, rot_dim=4, vdim=5, kv_rank=19, q_rank=9, window=30),          # a cached row of 23 columns
 ], vocab=101, width=44, mult=0.9)
 
 # rms(difference, mean taken off) / rms(logits, mean taken off) of a row may be at most this
