@@ -66,6 +66,8 @@ LIBRARIES: Dict[str, dict] = {
     "norm_gate": {"kind": "hip", "sources": ["kernels/norm_gate.hip"], "headers": ["kernels/common.h"]},
     "ssm": {"kind": "hip", "sources": ["kernels/ssm.hip"], "headers": ["kernels/common.h"]},
     "latent_attention": {"kind": "hip", "sources": ["kernels/latent_attention.hip"], "headers": ["kernels/common.h"]},
+    "scored_attention": {"kind": "hip", "sources": ["kernels/scored_attention.hip"], "headers": ["kernels/common.h"]},
+    "gated_recurrence": {"kind": "hip", "sources": ["kernels/gated_recurrence.hip"], "headers": ["kernels/common.h"]},
     "sampling": {"kind": "hip", "sources": ["kernels/sampling.hip"],
                  "headers": ["kernels/common.h", "kernels/noalloc.h"]},
     "peaks": {"kind": "hip", "sources": ["kernels/peaks.hip"], "headers": ["kernels/common.h"]},
@@ -73,13 +75,13 @@ LIBRARIES: Dict[str, dict] = {
     # (host code only; it calls the kernel libraries' entry points)
     "engine": {
         "kind": "hiphost",
-        "sources": ["engine/ops.cc", "engine/ops_sequence.cc", "engine/parts.cc", "engine/parts_gated.cc", "engine/mamba2.cc",
-                    "engine/latent_attention.cc", "engine/json.cc", "engine/weights.cc", "engine/arch.cc",
-                    "engine/gpt2.cc", "engine/kugulorn.cc", "engine/engine.cc", "engine/engine_api.cc"],
+        "sources": ["engine/ops.cc", "engine/ops_sequence.cc", "engine/ops_scored.cc", "engine/parts.cc", "engine/parts_gated.cc",
+                    "engine/mamba2.cc", "engine/latent_attention.cc", "engine/scored_attention.cc", "engine/recurrent_parts.cc", "engine/json.cc", "engine/weights.cc", "engine/arch.cc",
+                    "engine/gpt2.cc", "engine/kugulorn.cc", "engine/rekirax.cc", "engine/engine.cc", "engine/engine_api.cc"],
         "headers": ["engine/ops.h", "engine/parts.h", "engine/kernels.h", "engine/json.h", "engine/weights.h",
                     "engine/arch.h", "engine/engine.h", "runtime/cache_manager.h", "runtime/scheduler.h"],
         "needs": ["elementwise", "gemm_f32", "gemm_bf16", "attention", "attention_decode", "attention_prefill",
-                  "norm_gate", "ssm", "latent_attention", "sampling", "runtime"],
+                  "norm_gate", "ssm", "latent_attention", "scored_attention", "gated_recurrence", "sampling", "runtime"],
     },
     # the command line: a program, not a library (mini_llm_amd/_lib/mini-llm; bin/mini-llm starts it)
     "cli": {

@@ -20,6 +20,7 @@ void register_builtin_architectures() {
     std::call_once(once, [] {
         register_gpt2();
         register_kugulorn();
+        register_rekirax();
         if (const char* env = std::getenv("MINI_LLM_PLUGINS")) {
             std::stringstream ss(env);
             for (std::string path; std::getline(ss, path, ':');)

@@ -49,6 +49,7 @@ struct Architecture {
 void register_architecture(const Architecture& a, const std::string& model_type = "");
 void register_gpt2();              // gpt2.cc
 void register_kugulorn();          // kugulorn.cc
+void register_rekirax();           // rekirax.cc
 // Loads a shared library whose initialisers register parts and architectures (dlopen; stays loaded).
 // Also called for every path in the environment variable MINI_LLM_PLUGINS (colon-separated), once.
 void load_plugin(const std::string& path);

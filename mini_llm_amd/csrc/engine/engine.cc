@@ -39,7 +39,7 @@ void CacheStorage::allocate(const std::vector<CacheNeed>& needs, int n_pages, in
     std::vector<std::vector<int>> members;
     std::vector<int> group_of(needs.size(), -1);
     for (size_t c = 0; c < needs.size(); ++c) {
-        if (needs[c].kind != 1) continue;
+        if (!(needs[c].kind & 1)) continue;
         const Key k{needs[c].n_kv_heads, needs[c].head_dim, needs[c].value_dim < 0 ? needs[c].head_dim : needs[c].value_dim, needs[c].window};
         size_t g = 0;
         while (g < keys.size() && !(keys[g] == k)) ++g;
@@ -66,7 +66,7 @@ void CacheStorage::allocate(const std::vector<CacheNeed>& needs, int n_pages, in
         HIP_OK(hipMemset(pool, 0, std::max<size_t>(bytes, 16)));
         for (size_t j = 0; j < members[g].size(); ++j) {
             CacheView& v = views_[members[g][j]];
-            v.kind = 1;
+            v.kind |= 1;
             v.k_pages = Tensor2(static_cast<char*>(pool) + j * (k_bytes + v_bytes), dtype, rows, kv_dim);
             v.v_pages = v_dim > 0 ? Tensor2(static_cast<char*>(pool) + j * (k_bytes + v_bytes) + k_bytes, dtype, rows, v_dim) : Tensor2();
             v.group = static_cast<int>(g);
@@ -75,18 +75,29 @@ void CacheStorage::allocate(const std::vector<CacheNeed>& needs, int n_pages, in
             bytes_per_token_ += static_cast<size_t>(kv_dim + v_dim) * esz;
         }
     }
-    for (size_t c = 0; c < needs.size(); ++c) {
-        if (needs[c].kind != 2) continue;
-        void* state = nullptr;
-        const size_t bytes = needs[c].state_bytes * n_state_slots;
-        HIP_OK(hipMalloc(&state, std::max<size_t>(bytes, 16)));
-        allocations_.push_back(state);
+    // the states of all caches lie side by side in a request's slot: one allocation [slots][bytes of all states],
+    // which one kernel clears when a request begins
+    size_t slot_bytes = 0;
+    for (size_t c = 0; c < needs.size(); ++c)
+        if (needs[c].kind & 2) slot_bytes += (needs[c].state_bytes + 15) / 16 * 16;
+    if (slot_bytes > 0) {
+        const size_t bytes = slot_bytes * n_state_slots;
+        HIP_OK(hipMalloc(&state_, std::max<size_t>(bytes, 16)));
+        allocations_.push_back(state_);
         allocation_bytes_.push_back(bytes);
-        HIP_OK(hipMemset(state, 0, std::max<size_t>(bytes, 16)));
-        views_[c].kind = 2;
-        views_[c].state = state;
-        views_[c].slot_bytes = needs[c].state_bytes;
-        views_[c].n_slots = n_state_slots;
+        HIP_OK(hipMemset(state_, 0, std::max<size_t>(bytes, 16)));
+        state_slot_bytes_ = slot_bytes;
+        state_slots_ = n_state_slots;
+        size_t at = 0;
+        for (size_t c = 0; c < needs.size(); ++c) {
+            if (!(needs[c].kind & 2)) continue;
+            views_[c].kind |= 2;
+            views_[c].state = static_cast<char*>(state_) + at;
+            views_[c].slot_bytes = slot_bytes;
+            views_[c].state_bytes = needs[c].state_bytes;
+            views_[c].n_slots = n_state_slots;
+            at += (needs[c].state_bytes + 15) / 16 * 16;
+        }
     }
     manager_.reset(new CacheManager(group_specs_, n_state_slots));
 }
@@ -96,8 +107,7 @@ CacheStorage::~CacheStorage() {
 }
 
 void CacheStorage::reset_fresh_states(const StepView& step, hipStream_t s) const {
-    for (const CacheView& v : views_)
-        if (v.kind == 2) reset_state(v.state, v.slot_bytes, v.n_slots, step.state_slots, step.starts, step.n_seqs, s);
+    if (state_ != nullptr) reset_state(state_, state_slot_bytes_, state_slots_, step.state_slots, step.starts, step.n_seqs, s);
 }
 
 void CacheStorage::poison() {
@@ -112,7 +122,7 @@ static int pages_for_memory_fraction(const std::vector<CacheNeed>& needs, int dt
     if (fraction > 1.0) throw EngineError("kv_memory_fraction must be at most 1");
     size_t per_token = 0;
     for (const CacheNeed& n : needs)
-        if (n.kind == 1) per_token += static_cast<size_t>(n.n_kv_heads) * (n.head_dim + (n.value_dim < 0 ? n.head_dim : n.value_dim)) * dtype_size(dtype);
+        if (n.kind & 1) per_token += static_cast<size_t>(n.n_kv_heads) * (n.head_dim + (n.value_dim < 0 ? n.head_dim : n.value_dim)) * dtype_size(dtype);
     if (per_token == 0) return 1;
     size_t free_bytes = 0, total_bytes = 0;
     HIP_OK(hipMemGetInfo(&free_bytes, &total_bytes));

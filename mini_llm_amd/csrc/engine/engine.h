@@ -91,6 +91,9 @@ private:
     std::vector<size_t> allocation_bytes_;
     std::unique_ptr<CacheManager> manager_;
     size_t bytes_per_token_ = 0;
+    void* state_ = nullptr;            // [slots][the states of all caches side by side]
+    size_t state_slot_bytes_ = 0;
+    int state_slots_ = 0;
 };
 
 // A request's share of a step.

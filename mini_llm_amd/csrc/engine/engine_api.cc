@@ -350,7 +350,7 @@ int mllm_runner_info(void* runner, char* out, int cap) {
         j.set("n_requests", Json::of(r->manager().n_requests()));
         j.set("cache_bytes_per_token", Json::of(static_cast<int64_t>(r->cache().bytes_per_token())));
         int64_t state_bytes = 0;
-        for (const CacheNeed& n : m.caches) if (n.kind == 2) state_bytes += static_cast<int64_t>(n.state_bytes);
+        for (const CacheNeed& n : m.caches) if (n.kind & 2) state_bytes += static_cast<int64_t>(n.state_bytes);
         j.set("state_bytes_per_request", Json::of(state_bytes));
         j.set("weight_bytes", Json::of(c.weight_bytes));
         j.set("flops_per_token", Json::of(c.flops_per_token));

@@ -75,6 +75,9 @@ int mllm_fill_zero(void* p, size_t bytes, hipStream_t stream);
 int mllm_conv_silu(const float* proj, int ld, int col0, int C, const float* w, const float* bias, int taps,
                    const int* token_seq, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
                    float* out, int ldo, int T, int B, int write, hipStream_t stream);
+int mllm_conv_residual(const float* in, int ld, int C, const float* w, int taps, const int* token_seq, const int* cu_q,
+                       const int* state_slots, float* state, size_t slot_floats, void* out, int ldo, int out_dtype, int T,
+                       int B, int write, hipStream_t stream);
 int mllm_ssm_scan(const float* xbc, int ldx, const float* raw_dt, int ldd, const float* dt_bias, const float* A_log,
                   const float* Dskip, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
                   size_t scan_offset, float* y, int ldy, size_t part_stride, int T, int B, int max_q_len, int H, int P, int N,
@@ -97,6 +100,24 @@ int mllm_latent_attention_tiles(const void* qa, const void* k_pages, const void*
                                 float* partials, int single_tokens, hipStream_t stream);
 int mllm_latent_expand(const void* o_lat, int ldo, const void* w_uv, int ldw, void* out, int ldout, int T, int H, int Dv, int R,
                        int dtype, hipStream_t stream);
+
+// scored_attention.hip
+int mllm_qk_prepare(const float* proj, int ld, int q_col, int k_col, int v_col, int T, int H, int G, int d, int dv,
+                    int norm_mode, const float* wq, const float* wk, float eps, int rot_dims, double rot_base,
+                    const int* positions, const int* slots, void* q_out, int ldq, void* k_pages, void* v_pages, int dtype,
+                    hipStream_t stream);
+int mllm_scored_attention_rows(const void* q, int ldq, const void* k_pages, const void* v_pages, const int* block_tables,
+                               int max_blocks, const int* token_seq, const int* positions, int n_tokens, int H, int G, int d,
+                               int dv, int page_size, float scale, float softcap, int window, int chunk, const float* r1,
+                               const float* r2, const float* gate, int ldg, void* out, int ldo, int dtype, hipStream_t stream);
+
+// gated_recurrence.hip
+int mllm_hgrn2_parts(int d);
+int mllm_hgrn2_scan(const float* proj, int ld, int q_col, int f_col, int v_col, const float* f_bias, const float* lower,
+                    const int* cu_q, const int* state_slots, float* state, size_t slot_floats, size_t state_offset, float* y, int ldy,
+                    size_t part_stride, int T, int B, int H, int d, int dv, int write, hipStream_t stream);
+int mllm_concat_cast(const float* a, const float* b, int T, int D, void* out, int dtype, hipStream_t stream);
+int mllm_glu_act(const void* gu, int ld, int T, int F, int act, void* out, int ldo, int dtype, hipStream_t stream);
 
 // sampling.hip
 int mllm_argmax_chunks(int V);

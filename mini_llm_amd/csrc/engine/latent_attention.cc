@@ -71,7 +71,7 @@ public:
     void forward(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write, Arena& arena,
                  hipStream_t s) const override {
         const int E = sh_.kv_rank + sh_.rot_dim, T = step.n_tokens, g = cache.group, H = sh_.n_heads;
-        if (cache.kind != 1 || cache.k_pages.cols != E) fail("latent_attention needs pages of %d-wide rows", E);
+        if (!cache.has_pages() || cache.k_pages.cols != E) fail("latent_attention needs pages of %d-wide rows", E);
         if (write && !own_kv_) fail("a latent-attention layer without a key/value latent of its own cannot write a cache");
         Tensor2 dq = arena.tensor(F32, T, sh_.q_rank), cq = arena.tensor(dtype_, T, sh_.q_rank);
         const bool fill = own_kv_ && write;

@@ -49,7 +49,7 @@ public:
     }
     void forward(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write, Arena& arena,
                  hipStream_t s) const override {
-        if (cache.kind != 2 || cache.slot_bytes != slot_floats_ * 4) fail("mamba2 needs a state of %zu floats per request", slot_floats_);
+        if (!cache.has_state() || cache.state_bytes != slot_floats_ * 4) fail("mamba2 needs a state of %zu floats per request", slot_floats_);
         const int T = step.n_tokens, width = in_.out_features();
         // (rows padded to whole 16 bytes)
         Tensor2 proj(arena.take(static_cast<size_t>(T) * ((width + 3) / 4 * 4) * 4), F32, T, width, (width + 3) / 4 * 4);
@@ -57,7 +57,7 @@ public:
         StageTimes::get().mark("in_proj", s);
         StateArgs st;
         st.token_seq = step.token_seq; st.cu_q = step.cu_q; st.state_slots = step.state_slots; st.n_seqs = step.n_seqs;
-        st.state = static_cast<float*>(cache.state); st.slot_floats = slot_floats_; st.n_slots = cache.n_slots; st.write = write;
+        st.state = static_cast<float*>(cache.state); st.slot_floats = cache.slot_bytes / 4; st.n_slots = cache.n_slots; st.write = write;
         st.max_q_len = step.max_q_len;
         Tensor2 xbc = arena.tensor(F32, T, channels_);
         conv_silu(proj, inner_, conv_, conv_bias_, st, xbc, s);

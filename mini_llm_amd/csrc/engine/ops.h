@@ -236,6 +236,54 @@ size_t latent_attention_workspace_floats(int kv_rank);
 // out[t, h*value_dim + e] = sum_r w_uv[h*value_dim + e, r] * o_lat[t, h, r]
 void latent_expand(const Tensor2& o_lat, const Tensor2& w_uv, const Tensor2& out, const LatentShape& sh, hipStream_t stream);
 
+// -- attention with shaped scores -------------------------------------------------------------------
+// out = in + conv(in): a causal convolution per channel over `taps` inputs (taps [channels, taps], the last tap
+// the token's own), added onto its input; in fp32 [T, C], out in its own dtype. Carried inputs as for conv_silu.
+void conv_residual(const Tensor2& in, const Tensor2& weight, const StateArgs& st, const Tensor2& out, hipStream_t stream);
+// Sizes and constants of an attention whose scores are shaped before the softmax (kernels/scored_attention.hip).
+struct ScoredShape {
+    int n_heads = 0, n_kv_heads = 0, dim = 0, value_dim = 0;
+    float scale = 1.f, softcap = 0.f;          // softcap <= 0: none
+    int window = 0, chunk = 0;                 // sliding window or chunked causal mask; both 0: plain causal
+    const float* r1 = nullptr;                 // per head: s -= r1 ln(1 + r2 (i - j)); null: none
+    const float* r2 = nullptr;
+    int norm_mode = 0;                         // 0 none, 1 per head with one weight [dim], 2 over the whole row
+    const float* q_norm = nullptr;
+    const float* k_norm = nullptr;
+    float eps = 1e-6f;
+    int rot_dims = 0;                          // the first rot_dims columns of a head are turned (half-split pairs)
+    double rot_base = 10000.0;
+};
+// From the fp32 rows of the input projection (queries at q_col, keys at k_col, values at v_col; v_col < 0: the
+// values are the keys before their norm): q [T, heads * dim] normed and turned, and the keys and values written
+// to their page rows (slots[t]).
+void qk_prepare(const Tensor2& proj, int q_col, int k_col, int v_col, const ScoredShape& sh, const int* positions,
+                const int* slots, const Tensor2& q, const Tensor2& k_pages, const Tensor2& v_pages, hipStream_t stream);
+struct ScoredStep {
+    const int* block_tables = nullptr;     // [n_seqs, max_blocks]
+    int max_blocks = 0, n_seqs = 0, max_q_len = 0, max_ctx_len = 0, page_size = 0;
+    const int* token_seq = nullptr;        // [T]
+    const int* positions = nullptr;        // [T]
+    const int* cu_q = nullptr;             // [n_seqs + 1]
+    const int* ctx_len = nullptr;          // [n_seqs]
+};
+// out[t, h] = sum_j softmax_j(shaped score) v_j over the visible keys of the pages, times sigmoid(gate[t, gate_col +
+// h * value_dim ..]) if a gate (fp32 rows) is given.
+void scored_attention(const Tensor2& q, const Tensor2& k_pages, const Tensor2& v_pages, const ScoredStep& step,
+                      const ScoredShape& sh, const Tensor2* gate, int gate_col, const Tensor2& out, hipStream_t stream);
+
+// -- gated linear recurrence (HGRN2) ----------------------------------------------------------------
+// proj (fp32 rows): raw queries at q_col and raw gates at f_col (heads * dim each), values at v_col (heads * value_dim).
+// y: hgrn2_parts(dim) shares [T, heads * value_dim], y.rows * y.stride floats apart; the state ([heads][dim][value_dim]
+// fp32) lies state_offset floats into a request's slot.
+void hgrn2_scan(const Tensor2& proj, int q_col, int f_col, int v_col, const float* f_bias, const float* lower, const StateArgs& st,
+                size_t state_offset, int heads, int dim, int value_dim, const Tensor2& y, hipStream_t stream);
+int hgrn2_parts(int dim);
+// out = [a | b] row by row in out's dtype (a, b fp32 [T, D])
+void concat_cast(const Tensor2& a, const Tensor2& b, const Tensor2& out, hipStream_t stream);
+// out[t, j] = act(gu[t, j]) * gu[t, F + j] (act: GELU_TANH)
+void glu_act(const Tensor2& gu, int act, const Tensor2& out, hipStream_t stream);
+
 // `mirror` (optional): a second place for the chosen tokens, which may be pinned host memory (the kernel that
 // chooses writes it: no copy has to be launched for the host to read them).
 void argmax(const Tensor2& logits, int* out, hipStream_t stream, int* mirror = nullptr);

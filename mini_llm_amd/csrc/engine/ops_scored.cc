@@ -1,0 +1,139 @@
+// Checked dispatch of the attention with shaped scores, the gated linear recurrence, the convolution added
+// onto its input and their small companions (declared in ops.h beside the other ops).
+#include <algorithm>
+
+#include "kernels.h"
+#include "ops.h"
+
+namespace minillm {
+
+namespace {
+void check(int rc, const char* what) {
+    if (rc == 0) return;
+    if (rc < 0) fail("%s: the kernel refuses these sizes (code %d)", what, rc);
+    fail("%s: HIP error %d (%s) at launch", what, rc, hipGetErrorString(static_cast<hipError_t>(rc)));
+}
+void need_act(const Tensor2& t, const char* name) {
+    if (t.dtype != F32 && t.dtype != BF16) fail("%s: unsupported dtype code %d (float32 or bfloat16)", name, t.dtype);
+    if (t.data == nullptr && t.rows * t.cols > 0) fail("%s: null data pointer", name);
+}
+void need_f32(const Tensor2& t, const char* name) {
+    if (t.dtype != F32 || (t.data == nullptr && t.rows * t.cols > 0)) fail("%s must be float32", name);
+}
+int i32(int64_t v) { return static_cast<int>(v); }
+
+void check_state(const StateArgs& st, size_t floats_needed, const char* what) {
+    if (st.token_seq == nullptr || st.cu_q == nullptr || st.state_slots == nullptr || st.n_seqs < 1)
+        fail("%s: the step's token_seq, cu_q and state slots are needed", what);
+    if (st.state == nullptr || st.n_slots < 1 || st.slot_floats < floats_needed)
+        fail("%s: a state slot holds %zu floats, %zu are needed", what, st.slot_floats, floats_needed);
+}
+
+void check_shape(const ScoredShape& sh, const char* what) {
+    if (sh.n_heads < 1 || sh.n_kv_heads < 1 || sh.n_heads % sh.n_kv_heads != 0 || sh.dim < 1 || sh.value_dim < 1)
+        fail("%s: %d heads over %d key/value heads of %d / %d do not fit", what, sh.n_heads, sh.n_kv_heads, sh.dim, sh.value_dim);
+    if (sh.window < 0 || sh.chunk < 0 || (sh.window > 0 && sh.chunk > 0)) fail("%s: a window or a chunk, not both", what);
+    if ((sh.r1 != nullptr) != (sh.r2 != nullptr)) fail("%s: the distance bias needs both of its numbers per head", what);
+}
+}  // namespace
+
+void conv_residual(const Tensor2& in, const Tensor2& weight, const StateArgs& st, const Tensor2& out, hipStream_t stream) {
+    need_f32(in, "conv_residual: the input");
+    need_f32(weight, "conv_residual: the taps");
+    need_act(out, "conv_residual: out");
+    const int C = i32(weight.rows), taps = i32(weight.cols);
+    if (!weight.contiguous() || taps < 1 || taps > 16) fail("conv_residual: taps [channels, 1 to 16] contiguous are needed");
+    if (in.cols != C || out.cols != C || out.rows != in.rows) fail("conv_residual: input and out must be [T, %d]", C);
+    check_state(st, static_cast<size_t>(taps - 1) * C, "conv_residual");
+    check(mllm_conv_residual(static_cast<const float*>(in.data), i32(in.stride), C, static_cast<const float*>(weight.data), taps, st.token_seq,
+                             st.cu_q, st.state_slots, st.state, st.slot_floats, out.data, i32(out.stride), out.dtype, i32(in.rows), st.n_seqs,
+                             st.write ? 1 : 0, stream), "conv_residual");
+}
+
+void qk_prepare(const Tensor2& proj, int q_col, int k_col, int v_col, const ScoredShape& sh, const int* positions,
+                const int* slots, const Tensor2& q, const Tensor2& k_pages, const Tensor2& v_pages, hipStream_t stream) {
+    check_shape(sh, "qk_prepare");
+    need_f32(proj, "qk_prepare: the projection");
+    need_act(q, "qk_prepare: q");
+    const int64_t nq = static_cast<int64_t>(sh.n_heads) * sh.dim, nk = static_cast<int64_t>(sh.n_kv_heads) * sh.dim,
+                  nv = static_cast<int64_t>(sh.n_kv_heads) * sh.value_dim;
+    if (q_col < 0 || q_col + nq > proj.cols || k_col < 0 || k_col + nk > proj.cols || (v_col >= 0 && v_col + nv > proj.cols))
+        fail("qk_prepare: queries, keys or values lie outside the projection's rows of %lld", (long long)proj.cols);
+    if (v_col < 0 && sh.value_dim != sh.dim) fail("qk_prepare: values taken from the keys must have the keys' width");
+    if (q.rows != proj.rows || q.cols != nq) fail("qk_prepare: q must be [T, %lld]", (long long)nq);
+    if (k_pages.dtype != q.dtype || v_pages.dtype != q.dtype || !k_pages.contiguous() || !v_pages.contiguous() || k_pages.cols != nk ||
+        v_pages.cols != nv || k_pages.rows != v_pages.rows)
+        fail("qk_prepare: the pages must be contiguous [rows, %lld] and [rows, %lld] %s", (long long)nk, (long long)nv, dtype_name(q.dtype));
+    if (positions == nullptr || slots == nullptr) fail("qk_prepare: positions and page rows are needed");
+    if (sh.norm_mode < 0 || sh.norm_mode > 2 || (sh.norm_mode != 0 && (sh.q_norm == nullptr || sh.k_norm == nullptr)))
+        fail("qk_prepare: norm mode %d needs its two weights", sh.norm_mode);
+    if (sh.rot_dims < 0 || sh.rot_dims % 2 != 0 || sh.rot_dims > sh.dim || (sh.rot_dims > 0 && !(sh.rot_base > 0)))
+        fail("qk_prepare: %d turned columns of %d (even, at most the head) and a positive base are needed", sh.rot_dims, sh.dim);
+    check(mllm_qk_prepare(static_cast<const float*>(proj.data), i32(proj.stride), q_col, k_col, v_col, i32(proj.rows), sh.n_heads, sh.n_kv_heads,
+                          sh.dim, sh.value_dim, sh.norm_mode, sh.q_norm, sh.k_norm, sh.eps, sh.rot_dims, sh.rot_base, positions, slots, q.data,
+                          i32(q.stride), k_pages.data, v_pages.data, q.dtype, stream), "qk_prepare");
+}
+
+void scored_attention(const Tensor2& q, const Tensor2& k_pages, const Tensor2& v_pages, const ScoredStep& step,
+                      const ScoredShape& sh, const Tensor2* gate, int gate_col, const Tensor2& out, hipStream_t stream) {
+    check_shape(sh, "scored_attention");
+    need_act(q, "scored_attention: q");
+    const int64_t nq = static_cast<int64_t>(sh.n_heads) * sh.dim, nk = static_cast<int64_t>(sh.n_kv_heads) * sh.dim,
+                  nv = static_cast<int64_t>(sh.n_kv_heads) * sh.value_dim, no = static_cast<int64_t>(sh.n_heads) * sh.value_dim;
+    if (q.cols != nq) fail("scored_attention: q must be [T, %lld]", (long long)nq);
+    if (out.dtype != q.dtype || out.rows != q.rows || out.cols != no) fail("scored_attention: out must be [T, %lld] %s", (long long)no, dtype_name(q.dtype));
+    if (k_pages.dtype != q.dtype || v_pages.dtype != q.dtype || !k_pages.contiguous() || !v_pages.contiguous() || k_pages.cols != nk ||
+        v_pages.cols != nv || k_pages.rows != v_pages.rows)
+        fail("scored_attention: the pages must be contiguous [rows, %lld] and [rows, %lld] %s", (long long)nk, (long long)nv, dtype_name(q.dtype));
+    if (step.page_size < 1 || k_pages.rows % step.page_size != 0) fail("scored_attention: the page pool is not a whole number of pages");
+    if (step.block_tables == nullptr || step.token_seq == nullptr || step.positions == nullptr || step.max_blocks < 1)
+        fail("scored_attention: block tables, token_seq and positions are needed");
+    const float* g = nullptr;
+    int ldg = 0;
+    if (gate != nullptr) {
+        need_f32(*gate, "scored_attention: the gate");
+        if (gate->rows != q.rows || gate_col < 0 || gate_col + no > gate->cols) fail("scored_attention: the gate's columns lie outside its rows");
+        g = static_cast<const float*>(gate->data) + gate_col;
+        ldg = i32(gate->stride);
+    }
+    check(mllm_scored_attention_rows(q.data, i32(q.stride), k_pages.data, v_pages.data, step.block_tables, step.max_blocks, step.token_seq,
+                                     step.positions, i32(q.rows), sh.n_heads, sh.n_kv_heads, sh.dim, sh.value_dim, step.page_size, sh.scale,
+                                     sh.softcap, sh.window, sh.chunk, sh.r1, sh.r2, g, ldg, out.data, i32(out.stride), q.dtype, stream),
+          "scored_attention");
+}
+
+int hgrn2_parts(int dim) { return mllm_hgrn2_parts(dim); }
+
+void hgrn2_scan(const Tensor2& proj, int q_col, int f_col, int v_col, const float* f_bias, const float* lower, const StateArgs& st,
+                size_t state_offset, int heads, int dim, int value_dim, const Tensor2& y, hipStream_t stream) {
+    need_f32(proj, "hgrn2_scan: the projection");
+    need_f32(y, "hgrn2_scan: y");
+    if (heads < 1 || dim < 1 || value_dim < 1) fail("hgrn2_scan: heads and sizes must be positive");
+    const int64_t nq = static_cast<int64_t>(heads) * dim, nv = static_cast<int64_t>(heads) * value_dim;
+    if (q_col < 0 || q_col + nq > proj.cols || f_col < 0 || f_col + nq > proj.cols || v_col < 0 || v_col + nv > proj.cols)
+        fail("hgrn2_scan: queries, gates or values lie outside the projection's rows of %lld", (long long)proj.cols);
+    if (y.rows != proj.rows || y.cols != nv) fail("hgrn2_scan: y must be [%lld, %lld]", (long long)proj.rows, (long long)nv);
+    if (lower == nullptr) fail("hgrn2_scan: the gates' lower bounds are needed");
+    check_state(st, state_offset + static_cast<size_t>(heads) * dim * value_dim, "hgrn2_scan");
+    check(mllm_hgrn2_scan(static_cast<const float*>(proj.data), i32(proj.stride), q_col, f_col, v_col, f_bias, lower, st.cu_q, st.state_slots,
+                          st.state, st.slot_floats, state_offset, static_cast<float*>(y.data), i32(y.stride), static_cast<size_t>(y.rows) * y.stride,
+                          i32(proj.rows), st.n_seqs, heads, dim, value_dim, st.write ? 1 : 0, stream), "hgrn2_scan");
+}
+
+void concat_cast(const Tensor2& a, const Tensor2& b, const Tensor2& out, hipStream_t stream) {
+    need_f32(a, "concat_cast: a");
+    need_f32(b, "concat_cast: b");
+    need_act(out, "concat_cast: out");
+    if (!a.contiguous() || !b.contiguous() || !out.contiguous() || a.rows != b.rows || a.cols != b.cols || out.rows != a.rows || out.cols != 2 * a.cols)
+        fail("concat_cast: a and b must be contiguous [T, D] and out [T, 2 D]");
+    check(mllm_concat_cast(static_cast<const float*>(a.data), static_cast<const float*>(b.data), i32(a.rows), i32(a.cols), out.data, out.dtype, stream),
+          "concat_cast");
+}
+
+void glu_act(const Tensor2& gu, int act, const Tensor2& out, hipStream_t stream) {
+    need_act(gu, "glu_act: the input");
+    if (out.dtype != gu.dtype || out.rows != gu.rows || gu.cols != 2 * out.cols) fail("glu_act: out must be [T, F] for an input of [T, 2 F], of one dtype");
+    check(mllm_glu_act(gu.data, i32(gu.stride), i32(gu.rows), i32(out.cols), act, out.data, i32(out.stride), gu.dtype, stream), "glu_act");
+}
+
+}  // namespace minillm

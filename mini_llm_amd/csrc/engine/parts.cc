@@ -108,6 +108,10 @@ void Norm::linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int e
     lin(h, out, epilogue, kv, s);
 }
 
+void Norm::forward_into(const Tensor2&, const int*, const Tensor2&, hipStream_t) const {
+    fail("this kind of norm cannot write into a tensor it is handed");
+}
+
 void Norm::add_scaled(const Tensor2&, const float*, float, const Tensor2&, bool, hipStream_t) const {
     fail("this kind of norm cannot stand behind a sub-layer (it has no scaled add)");
 }
@@ -190,7 +194,7 @@ public:
     }
     void forward(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write, Arena& arena,
                  hipStream_t s) const override {
-        if (cache.kind != 1) fail("attention needs a cache of pages");
+        if (!cache.has_pages()) fail("attention needs a cache of pages");
         const int T = step.n_tokens, g = cache.group;
         Tensor2 qkv = arena.tensor(dtype_, T, q_dim_ + 2 * kv_dim_);
         // Prompt portions: the QKV product is asked to put the new keys and values into the pages (how
@@ -304,19 +308,46 @@ private:
 
 // x += mixer(norm1(x)); x += feed_forward(norm2(x)): the norm stands before each sub-layer, on the
 // residual stream (/root/reference/src/model/gpt2_model.cu:279-363).
+// With the tensor "mixer_conv" ([width, taps] fp32) what the mixer reads is h + conv(h), h = norm1(x): a causal
+// convolution over time on each channel, the last tap the token's own; the last taps - 1 rows of h are carried
+// per request in the front of the layer's state slot (the mixer's own state, if it has one, lies behind them).
 class PreNormBlock final : public Block {
 public:
-    PreNormBlock(std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> norms)
+    PreNormBlock(std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> norms, const Params& p)
         : mixer_(std::move(m)), ff_(std::move(f)) {
         if (!mixer_) fail("a pre-norm block needs a mixer");
         if (norms.size() != (ff_ ? 2u : 1u)) fail("a pre-norm block has one norm per sub-layer (%d here), got %zu", ff_ ? 2 : 1, norms.size());
         norm1_ = std::move(norms[0]);
         if (ff_) norm2_ = std::move(norms[1]);
+        if (const Tensor2* c = p.weights_or_null("mixer_conv")) {
+            if (c->dtype != F32 || !c->contiguous() || c->cols < 1 || c->cols > 16) fail("a block's input convolution must be contiguous float32 [width, 1 to 16 taps]");
+            conv_ = *c;
+            conv_bytes_ = static_cast<size_t>(conv_.cols - 1) * conv_.rows * 4;
+            dtype_ = p.integer("dtype");
+        }
     }
     void forward(const Tensor2& x, const StepView& step, const CacheView& cache, bool write, Arena& arena,
                  hipStream_t s) const override {
         size_t mark = arena.mark();
-        {
+        if (conv_.data != nullptr) {
+            if (!cache.has_state() || cache.state_bytes < conv_bytes_) fail("a block with an input convolution needs %zu bytes of state per request", conv_bytes_);
+            if (x.cols != conv_.rows) fail("the input convolution has %lld channels, the stream %lld", (long long)conv_.rows, (long long)x.cols);
+            Tensor2 hn = arena.tensor(F32, x.rows, x.cols);      // the convolution reads the normed rows in fp32
+            norm1_->forward_into(x, nullptr, hn, s);
+            Tensor2 hc = arena.tensor(dtype_, x.rows, x.cols);
+            StateArgs st;
+            st.token_seq = step.token_seq; st.cu_q = step.cu_q; st.state_slots = step.state_slots; st.n_seqs = step.n_seqs;
+            st.max_q_len = step.max_q_len; st.state = static_cast<float*>(cache.state); st.slot_floats = cache.slot_bytes / 4;
+            st.n_slots = cache.n_slots; st.write = write;
+            conv_residual(hn, conv_, st, hc, s);
+            StageTimes::get().mark("input_conv", s);
+            CacheView rest = cache;                     // what lies behind the carried rows is the mixer's
+            rest.state = static_cast<char*>(cache.state) + conv_bytes_;
+            rest.state_bytes = cache.state_bytes - conv_bytes_;
+            if (rest.state_bytes == 0) rest.kind &= ~2;
+            NormedInput h(hc);
+            mixer_->forward(h, step, rest, x, write, arena, s);
+        } else {
             NormedInput h(*norm1_, x);
             mixer_->forward(h, step, cache, x, write, arena, s);
         }
@@ -329,10 +360,15 @@ public:
         arena.release(mark);
     }
     size_t workspace_bytes(int tokens) const override {
-        const size_t a = mixer_->workspace_bytes(tokens) + 2 * norm1_->workspace_bytes(tokens);
+        size_t a = mixer_->workspace_bytes(tokens) + 2 * norm1_->workspace_bytes(tokens);
+        if (conv_.data != nullptr) a += static_cast<size_t>(tokens) * conv_.rows * 8 + 1024;
         return ff_ ? std::max(a, ff_->workspace_bytes(tokens) + 2 * norm2_->workspace_bytes(tokens)) : a;
     }
-    CacheNeed cache_need() const override { return mixer_->cache_need(); }
+    CacheNeed cache_need() const override {
+        CacheNeed n = mixer_->cache_need();
+        if (conv_bytes_ > 0) { n.kind |= 2; n.state_bytes += conv_bytes_; }
+        return n;
+    }
     void reserve(int max_seqs, hipStream_t s) const override {
         mixer_->reserve(max_seqs, s);
         if (ff_) ff_->reserve(max_seqs, s);
@@ -341,12 +377,16 @@ public:
         norm1_->add_cost(c);
         mixer_->add_cost(c);
         if (ff_) { norm2_->add_cost(c); ff_->add_cost(c); }
+        if (conv_.data != nullptr) { c.weight_bytes += 4.0 * conv_.rows * conv_.cols; c.flops_per_token += 2.0 * conv_.rows * conv_.cols; }
     }
 
 private:
     std::unique_ptr<Mixer> mixer_;
     std::unique_ptr<FeedForward> ff_;
     std::unique_ptr<Norm> norm1_, norm2_;
+    Tensor2 conv_;                 // [width, taps], or empty: no input convolution
+    size_t conv_bytes_ = 0;
+    int dtype_ = BF16;
 };
 
 // Learned absolute positions: row pos[t] of a table is added to the token's embedding, in the embedding
@@ -426,6 +466,7 @@ Registry<NormFactory>& norms() { static Registry<NormFactory> r{"norm", {}}; ret
 Registry<MixerFactory>& mixers() { static Registry<MixerFactory> r{"mixer", {}}; return r; }
 Registry<FeedForwardFactory>& feed_forwards() { static Registry<FeedForwardFactory> r{"feed-forward", {}}; return r; }
 Registry<BlockFactory>& blocks() { static Registry<BlockFactory> r{"block arrangement", {}}; return r; }
+Registry<StreamStepFactory>& stream_steps() { static Registry<StreamStepFactory> r{"stream step", {}}; return r; }
 
 void register_builtin_parts() {
     static bool done = false;
@@ -437,12 +478,14 @@ void register_builtin_parts() {
     norms().kinds["layernorm"] = [](const Params& p) { return std::unique_ptr<Norm>(new LayerNorm(p)); };
     mixers().kinds["causal_attention"] = [](const Params& p) { return std::unique_ptr<Mixer>(new CausalSelfAttention(p)); };
     feed_forwards().kinds["dense_mlp"] = [](const Params& p) { return std::unique_ptr<FeedForward>(new DenseMLP(p)); };
-    blocks().kinds["pre_norm"] = [](std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> n, const Params&) {
-        return std::unique_ptr<Block>(new PreNormBlock(std::move(m), std::move(f), std::move(n)));
+    blocks().kinds["pre_norm"] = [](std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f, std::vector<std::unique_ptr<Norm>> n, const Params& p) {
+        return std::unique_ptr<Block>(new PreNormBlock(std::move(m), std::move(f), std::move(n), p));
     };
     register_gated_parts();
     register_mamba2();
     register_latent_attention();
+    register_scored_attention();
+    register_recurrent_parts();
 }
 }  // namespace
 
@@ -453,6 +496,7 @@ void register_norm(const std::string& kind, NormFactory f) { register_builtin_pa
 void register_mixer(const std::string& kind, MixerFactory f) { register_builtin_parts(); mixers().kinds[kind] = std::move(f); }
 void register_feed_forward(const std::string& kind, FeedForwardFactory f) { register_builtin_parts(); feed_forwards().kinds[kind] = std::move(f); }
 void register_block(const std::string& kind, BlockFactory f) { register_builtin_parts(); blocks().kinds[kind] = std::move(f); }
+void register_stream_step(const std::string& kind, StreamStepFactory f) { register_builtin_parts(); stream_steps().kinds[kind] = std::move(f); }
 
 bool has_part(const std::string& category, const std::string& kind) {
     register_builtin_parts();
@@ -463,6 +507,7 @@ bool has_part(const std::string& category, const std::string& kind) {
     if (category == "mixer") return mixers().kinds.count(kind) != 0;
     if (category == "feed_forward") return feed_forwards().kinds.count(kind) != 0;
     if (category == "block") return blocks().kinds.count(kind) != 0;
+    if (category == "stream_step") return stream_steps().kinds.count(kind) != 0;
     return false;
 }
 
@@ -490,6 +535,10 @@ std::unique_ptr<FeedForward> build_feed_forward(const std::string& kind, const P
     register_builtin_parts();
     return feed_forwards().get(kind)(p);
 }
+std::unique_ptr<StreamStep> build_stream_step(const std::string& kind, const Params& p) {
+    register_builtin_parts();
+    return stream_steps().get(kind)(p);
+}
 std::unique_ptr<Block> build_block(const std::string& kind, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
                                    std::vector<std::unique_ptr<Norm>> n, const Params& params) {
     register_builtin_parts();
@@ -502,8 +551,9 @@ std::unique_ptr<Block> build_block(const std::string& kind, std::unique_ptr<Mixe
 static void check_order(const DecoderModel& m) {
     if (!m.embedding || !m.head || !m.final_norm) fail("a model needs an embedding, a final norm and a head");
     for (const LayerCall& c : m.order)
-        if (c.layer < 0 || c.layer >= static_cast<int>(m.layers.size()) || c.cache < 0)
-            fail("the execution order names layer %d / cache %d, the model has %zu layers", c.layer, c.cache, m.layers.size());
+        if (c.layer < 0 || c.layer >= static_cast<int>(m.layers.size()) || c.cache < 0 || c.before >= static_cast<int>(m.stream_steps.size()))
+            fail("the execution order names layer %d / cache %d / stream step %d, the model has %zu layers and %zu stream steps", c.layer,
+                 c.cache, c.before, m.layers.size(), m.stream_steps.size());
 }
 
 std::vector<CacheNeed> DecoderModel::cache_needs() const {
@@ -527,13 +577,14 @@ std::vector<CacheNeed> DecoderModel::cache_needs() const {
             mine.value_dim != theirs.value_dim || mine.state_bytes != theirs.state_bytes)
             fail("layer %d reads cache %d, which another kind of mixer writes", c.layer, c.cache);
         // the pages are kept for the widest window among the calls that read them (0: every key)
-        if (theirs.kind == 1 && theirs.window > 0) needs[c.cache].window = mine.window > 0 ? std::max(theirs.window, mine.window) : 0;
+        if ((theirs.kind & 1) && theirs.window > 0) needs[c.cache].window = mine.window > 0 ? std::max(theirs.window, mine.window) : 0;
     }
     return needs;
 }
 
 void DecoderModel::reserve(int max_seqs, hipStream_t s) const {
     for (const auto& l : layers) l->reserve(max_seqs, s);
+    for (const auto& st : stream_steps) st->reserve(max_seqs, s);
     reserve_linear_scratch(s);
 }
 
@@ -549,6 +600,13 @@ StepCost DecoderModel::cost() const {
         seen[call.layer] = true;
         c.flops_per_token += one.flops_per_token;
         c.attention_flops_per_key += one.attention_flops_per_key;
+        if (call.before >= 0) {
+            // (a stream step's weights are read once per run of it; they are small and counted once)
+            StepCost st;
+            stream_steps[call.before]->add_cost(st);
+            if (call.pass == 0) c.weight_bytes += st.weight_bytes;
+            c.flops_per_token += st.flops_per_token;
+        }
     }
     final_norm->add_cost(c);
     head->add_cost(c);
@@ -560,8 +618,13 @@ size_t DecoderModel::workspace_bytes(int tokens, int n_logits) const {
     size_t per_layer = 0;
     for (const auto& l : layers) per_layer = std::max(per_layer, l->workspace_bytes(tokens));
     size_t stream = static_cast<size_t>(tokens) * hidden_size() * 4 + 256;
+    const size_t one = stream;
     for (const auto& l : layers)
-        if (l->wants_zeroed_rows()) { stream *= 2; break; }
+        if (l->wants_zeroed_rows()) { stream += one; break; }
+    for (const auto& st : stream_steps) {
+        if (st->wants_embedding_output()) { stream += one; break; }
+    }
+    for (const auto& st : stream_steps) per_layer = std::max(per_layer, st->workspace_bytes(tokens));
     const int rows = std::max(n_logits, 1);
     const size_t at_head = head->workspace_bytes(rows) + 2 * final_norm->workspace_bytes(rows);
     return stream + std::max(per_layer, at_head) + 4096;
@@ -575,6 +638,15 @@ void DecoderModel::forward(const StepView& step, const std::vector<CacheView>& c
     times.begin_step(step.max_q_len == 1 ? "decode" : (step.n_single > 0 ? "mixed" : "prefill"), step.n_seqs, step.n_tokens, s);
     Tensor2 x = arena.tensor(F32, step.n_tokens, hidden_size());
     embedding->forward(step, position.get(), x, s);
+    // a stream step that mixes the embedding's output back in later: a copy of it stays for the step
+    Tensor2 x0;
+    for (const auto& st : stream_steps) {
+        if (!st->wants_embedding_output()) continue;
+        x0 = arena.tensor(F32, step.n_tokens, hidden_size());
+        if (hipMemcpyAsync(x0.data, x.data, static_cast<size_t>(step.n_tokens) * hidden_size() * 4, hipMemcpyDeviceToDevice, s) != hipSuccess)
+            fail("the copy of the embedding's output failed");
+        break;
+    }
     times.mark("embed", s);
     StepView with_rows = step;
     for (const auto& l : layers) {
@@ -588,6 +660,12 @@ void DecoderModel::forward(const StepView& step, const std::vector<CacheView>& c
         if (c.cache >= static_cast<int>(caches.size()))
             fail("the execution order names cache %d, the step brings %zu caches", c.cache, caches.size());
         times.set_layer(c.layer);
+        if (c.before >= 0) {
+            const size_t mark = arena.mark();
+            stream_steps[c.before]->forward(x, x0, c.pass, with_rows, arena, s);
+            arena.release(mark);
+            times.mark("stream_step", s);
+        }
         layers[c.layer]->forward(x, with_rows, caches[c.cache], c.write, arena, s);
     }
     times.set_layer(-1);

@@ -103,17 +103,20 @@ struct StepView {
 
 // What a call of the execution order sees of its cache.
 struct CacheView {
-    int kind = 0;                  // 0 none, 1 pages of keys and values, 2 fixed-size state slots
+    int kind = 0;                  // bits: 1 pages of keys and values, 2 fixed-size state slots (3: both)
     Tensor2 k_pages, v_pages;      // [n_pages * page_size, kv_dim]
     int group = 0, page_size = 0, window = 0;
-    void* state = nullptr;         // [n_slots, slot_bytes]
-    size_t slot_bytes = 0;
+    void* state = nullptr;         // this cache's state in slot 0; slot i lies i * slot_bytes further on
+    size_t slot_bytes = 0;         // bytes between a slot and the next (the states of all caches lie side by side in a slot)
+    size_t state_bytes = 0;        // bytes of a slot that are this cache's own
     int n_slots = 0;
+    bool has_pages() const { return (kind & 1) != 0; }
+    bool has_state() const { return (kind & 2) != 0; }
 };
 
 // What a cache of the execution order asks of the cache manager: said by the mixer that writes it.
 struct CacheNeed {
-    int kind = 0;                        // 1 keys and values in pages, 2 fixed-size state, 0 none
+    int kind = 0;                        // bits: 1 keys and values in pages, 2 fixed-size state (3: both), 0 none
     int n_kv_heads = 0, head_dim = 0, window = 0;
     int value_dim = -1;                  // width of a head's value rows; -1: as the keys; 0: the pages hold key rows only
     size_t state_bytes = 0;
@@ -128,6 +131,7 @@ struct StepCost {
 };
 
 class PositionEncoding;
+class Mixer;
 
 // A bag of parameters a part is built from.
 struct Params {
@@ -135,6 +139,7 @@ struct Params {
     std::map<std::string, std::string> str;
     std::map<std::string, Tensor2> tensor;
     std::shared_ptr<const PositionEncoding> position;      // the model's position encoding, for mixers that take one
+    std::vector<std::shared_ptr<const Mixer>> mixers;      // mixers that a mixer made of others runs side by side
 
     double number(const std::string& key) const;
     double number(const std::string& key, double fallback) const;
@@ -197,6 +202,9 @@ public:
     virtual ~Norm() = default;
     // h[i,:] = norm(x[rows ? rows[i] : i, :]), n rows, from the arena
     virtual Tensor2 forward(const Tensor2& x, const int* rows, int n, Arena& arena, hipStream_t s) const = 0;
+    // out[i,:] = norm(x[rows ? rows[i] : i, :]) into a tensor of the caller's (any activation dtype; out may be x
+    // itself when rows is null and both are fp32). A norm without it refuses.
+    virtual void forward_into(const Tensor2& x, const int* rows, const Tensor2& out, hipStream_t s) const;
     // out = epilogue(lin(norm(x[rows]))); a norm with a fused kernel overrides this
     // (kv: a key/value scatter of the linear map, passed through to it)
     virtual void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,
@@ -262,6 +270,19 @@ public:
     virtual void add_cost(StepCost&) const = 0;
 };
 
+// Something that happens to the whole stream between two layers (an entry of the execution order names it
+// with `before`): x is the stream, x0 the embedding's output of the same step, `pass` the number the entry gives
+// (a group of layers that runs several times counts its runs).
+class StreamStep {
+public:
+    virtual ~StreamStep() = default;
+    virtual void forward(const Tensor2& x, const Tensor2& x0, int pass, const StepView& step, Arena& arena, hipStream_t s) const = 0;
+    virtual size_t workspace_bytes(int tokens) const = 0;
+    virtual bool wants_embedding_output() const { return false; }
+    virtual void reserve(int max_seqs, hipStream_t s) const { (void)max_seqs; (void)s; }
+    virtual void add_cost(StepCost&) const {}
+};
+
 // The stream's wanted rows to fp32 logits.
 class Head {
 public:
@@ -281,6 +302,7 @@ using HeadFactory = std::function<std::unique_ptr<Head>(const Params&)>;
 using NormFactory = std::function<std::unique_ptr<Norm>(const Params&)>;
 using MixerFactory = std::function<std::unique_ptr<Mixer>(const Params&)>;
 using FeedForwardFactory = std::function<std::unique_ptr<FeedForward>(const Params&)>;
+using StreamStepFactory = std::function<std::unique_ptr<StreamStep>(const Params&)>;
 // (the parameters are the arrangement's own: scales, multipliers; "pre_norm" has none)
 using BlockFactory = std::function<std::unique_ptr<Block>(std::unique_ptr<Mixer>, std::unique_ptr<FeedForward>,
                                                          std::vector<std::unique_ptr<Norm>>, const Params&)>;
@@ -291,7 +313,8 @@ void register_norm(const std::string& kind, NormFactory f);
 void register_mixer(const std::string& kind, MixerFactory f);
 void register_feed_forward(const std::string& kind, FeedForwardFactory f);
 void register_block(const std::string& kind, BlockFactory f);
-// category: position | embedding | head | norm | mixer | feed_forward | block
+void register_stream_step(const std::string& kind, StreamStepFactory f);
+// category: position | embedding | head | norm | mixer | feed_forward | block | stream_step
 bool has_part(const std::string& category, const std::string& kind);
 std::shared_ptr<const PositionEncoding> build_position(const std::string& kind, const Params& p);
 std::unique_ptr<Embedding> build_embedding(const std::string& kind, const Params& p);
@@ -299,6 +322,7 @@ std::unique_ptr<Head> build_head(const std::string& kind, const Params& p);
 std::unique_ptr<Norm> build_norm(const std::string& kind, const Params& p);
 std::unique_ptr<Mixer> build_mixer(const std::string& kind, const Params& p);
 std::unique_ptr<FeedForward> build_feed_forward(const std::string& kind, const Params& p);
+std::unique_ptr<StreamStep> build_stream_step(const std::string& kind, const Params& p);
 // (the feed-forward may be null: a layer without one; the norms are those of the sub-layers that exist)
 std::unique_ptr<Block> build_block(const std::string& kind, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
                                    std::vector<std::unique_ptr<Norm>> norms, const Params& params = Params());
@@ -308,11 +332,18 @@ std::unique_ptr<Block> build_block(const std::string& kind, std::unique_ptr<Mixe
 void register_gated_parts();
 void register_mamba2();
 void register_latent_attention();
+// Attention with shaped scores (scored_attention.cc); the gated linear recurrence, mixers side by side, the gated
+// feed-forward with biases, the embedding with a norm, the stream step that mixes the embedding's output back in
+// (recurrent_parts.cc).
+void register_scored_attention();
+void register_recurrent_parts();
 
 // One entry of the execution order: which layer runs, on which cache, and whether it writes it.
 struct LayerCall {
     int layer = 0, cache = 0;
     bool write = true;
+    int before = -1;               // >= 0: this stream step runs on the stream right before the layer
+    int pass = 0;                  // handed to that stream step
 };
 
 // A decoder-only model: the embedding (with the position encoding's table, if it has one), the calls
@@ -322,6 +353,7 @@ public:
     std::unique_ptr<Embedding> embedding;
     std::shared_ptr<const PositionEncoding> position;     // may be null: no position encoding
     std::vector<std::unique_ptr<Block>> layers;
+    std::vector<std::unique_ptr<StreamStep>> stream_steps;
     std::vector<LayerCall> order;
     std::unique_ptr<Norm> final_norm;
     std::unique_ptr<Head> head;

@@ -28,6 +28,10 @@ public:
         rmsnorm(x, weight_, eps_, 1, nullptr, h, rows, s);
         return h;
     }
+    void forward_into(const Tensor2& x, const int* rows, const Tensor2& out, hipStream_t s) const override {
+        if (x.cols != size_) fail("rmsnorm: rows of %lld, the norm is %d wide", (long long)x.cols, size_);
+        rmsnorm(x, weight_, eps_, 1, nullptr, out, rows, s);
+    }
     void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,
                 const KvScatter* kv, Arena& arena, hipStream_t s) const override {
         if (kv != nullptr) { Norm::linear(x, lin, out, epilogue, rows, kv, arena, s); return; }

@@ -1,0 +1,114 @@
+// Softmax attention whose scores are shaped before the softmax, as one mixer with its choices as parameters.
+#include "parts.h"
+
+namespace minillm {
+
+namespace {
+
+const float* f32_vector(const Params& p, const char* key, int64_t n) {
+    const Tensor2& t = p.weights(key);
+    if (t.dtype != F32 || t.rows * t.cols != n || !t.contiguous()) fail("scored_attention: '%s' must be contiguous float32 [%lld]", key, (long long)n);
+    return static_cast<const float*>(t.data);
+}
+
+// With h the mixer's input and one joined input projection whose rows are [queries: heads * dim | keys: kv_heads * dim |
+// values: kv_heads * value_dim (absent with values_from_keys) | gate: heads * value_dim (only with gated)]:
+//   q, k   RMS-normed (qk_norm "head": per head, one weight [dim] shared by the heads; "row": over all heads at once,
+//          weights as wide as the projections; "none"), then the first rot_dims columns of every head turned by the
+//          token's position (column i pairs with i + rot_dims / 2, angle p * rot_base^(-2i / rot_dims))
+//   v      its own projection, or (values_from_keys) the keys as projected, before their norm
+//   score  scale (q . k);  softcap > 0: softcap tanh(score / softcap);  with r1, r2 (one number per head each):
+//          minus r1 ln(1 + r2 (i - j))
+//   mask   causal, within a sliding window (0 <= i - j < window) or within the chunk of `chunk` positions that holds i
+//   out    W_o (concat_heads(softmax(score) v) * sigmoid(gate)), added into the stream.
+// Query head h reads key/value head h / (heads / kv_heads). Normed and turned keys and the values live in pages.
+// Parameters: heads, kv_heads, dim, value_dim, scale, softcap, window, chunk, rot_dims, rot_base, eps, dtype,
+// values_from_keys, gated; string qk_norm; tensors in.weight, out.weight, [q.norm, k.norm], [r1, r2].
+class ScoredAttention final : public Mixer {
+public:
+    explicit ScoredAttention(const Params& p) {
+        sh_.n_heads = p.integer("heads");
+        sh_.n_kv_heads = p.integer("kv_heads");
+        sh_.dim = p.integer("dim");
+        sh_.value_dim = p.integer("value_dim");
+        sh_.scale = static_cast<float>(p.number("scale"));
+        sh_.softcap = static_cast<float>(p.number("softcap", 0.0));
+        sh_.window = static_cast<int>(p.number("window", 0));
+        sh_.chunk = static_cast<int>(p.number("chunk", 0));
+        sh_.rot_dims = static_cast<int>(p.number("rot_dims", 0));
+        sh_.rot_base = p.number("rot_base", 10000.0);
+        sh_.eps = static_cast<float>(p.number("eps", 1e-6));
+        dtype_ = p.integer("dtype");
+        values_from_keys_ = p.number("values_from_keys", 0) != 0;
+        gated_ = p.number("gated", 0) != 0;
+        const int H = sh_.n_heads, G = sh_.n_kv_heads, d = sh_.dim, dv = sh_.value_dim;
+        if (H < 1 || G < 1 || H % G != 0 || d < 1 || dv < 1) fail("scored_attention: %d heads over %d key/value heads of %d / %d do not fit", H, G, d, dv);
+        if (sh_.window < 0 || sh_.chunk < 0 || (sh_.window > 0 && sh_.chunk > 0)) fail("scored_attention: a window or a chunk, not both");
+        if (values_from_keys_ && dv != d) fail("scored_attention: values taken from the keys have the keys' width, %d, not %d", d, dv);
+        if (sh_.rot_dims < 0 || sh_.rot_dims % 2 != 0 || sh_.rot_dims > d) fail("scored_attention: %d turned columns of %d: even and at most the head", sh_.rot_dims, d);
+        const std::string& mode = p.string("qk_norm");
+        if (mode == "none") sh_.norm_mode = 0;
+        else if (mode == "head") sh_.norm_mode = 1;
+        else if (mode == "row") sh_.norm_mode = 2;
+        else fail("scored_attention: qk_norm '%s' is not one of none, head, row", mode.c_str());
+        if (sh_.norm_mode == 1) { sh_.q_norm = f32_vector(p, "q.norm", d); sh_.k_norm = f32_vector(p, "k.norm", d); }
+        if (sh_.norm_mode == 2) { sh_.q_norm = f32_vector(p, "q.norm", static_cast<int64_t>(H) * d); sh_.k_norm = f32_vector(p, "k.norm", static_cast<int64_t>(G) * d); }
+        if (p.weights_or_null("r1") != nullptr) { sh_.r1 = f32_vector(p, "r1", H); sh_.r2 = f32_vector(p, "r2", H); }
+        in_ = Linear(p.weights("in.weight"), nullptr);
+        out_ = Linear(p.weights("out.weight"), nullptr);
+        k_col_ = H * d;
+        v_col_ = values_from_keys_ ? -1 : k_col_ + G * d;
+        gate_col_ = k_col_ + G * d + (values_from_keys_ ? 0 : G * dv);
+        if (in_.out_features() != gate_col_ + (gated_ ? H * dv : 0) || out_.in_features() != H * dv)
+            fail("scored_attention: the projections' shapes do not fit %d heads of %d / %d over %d key/value heads", H, d, dv, G);
+    }
+    void forward(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write, Arena& arena,
+                 hipStream_t s) const override {
+        if (!cache.has_pages()) fail("scored_attention needs a cache of pages");
+        if (!write) fail("scored_attention writes its own keys and values: it cannot read another call's cache");
+        const int T = step.n_tokens, g = cache.group, N = in_.out_features(), ld = (N + 3) / 4 * 4;
+        Tensor2 proj(arena.take(static_cast<size_t>(T) * ld * 4), F32, T, N, ld);
+        h.linear(in_, proj, STORE_F32, nullptr, arena, s);
+        Tensor2 q = arena.tensor(dtype_, T, sh_.n_heads * sh_.dim);
+        qk_prepare(proj, 0, k_col_, v_col_, sh_, step.positions, step.slots[g], q, cache.k_pages, cache.v_pages, s);
+        StageTimes::get().mark("qkv", s);
+        ScoredStep st;
+        st.block_tables = step.block_tables[g]; st.max_blocks = step.max_blocks[g]; st.n_seqs = step.n_seqs; st.max_q_len = step.max_q_len;
+        st.max_ctx_len = step.max_ctx_len; st.page_size = cache.page_size; st.token_seq = step.token_seq; st.positions = step.positions;
+        st.cu_q = step.cu_q; st.ctx_len = step.ctx_len;
+        Tensor2 o = arena.tensor(dtype_, T, sh_.n_heads * sh_.value_dim);
+        scored_attention(q, cache.k_pages, cache.v_pages, st, sh_, gated_ ? &proj : nullptr, gate_col_, o, s);
+        StageTimes::get().mark("attention", s);
+        out_(o, x, ADD_RESIDUAL, nullptr, s);
+        StageTimes::get().mark("out_proj", s);
+    }
+    size_t workspace_bytes(int tokens) const override {
+        return static_cast<size_t>(tokens) * ((in_.out_features() + 4) * 4 + (sh_.n_heads * (sh_.dim + sh_.value_dim) + in_.in_features()) * dtype_size(dtype_)) + 4096;
+    }
+    CacheNeed cache_need() const override {
+        CacheNeed n;
+        // (a chunked mask keeps its pages: only a sliding window tells the manager what it may take back)
+        n.kind = 1; n.n_kv_heads = sh_.n_kv_heads; n.head_dim = sh_.dim; n.value_dim = sh_.value_dim; n.window = sh_.window;
+        return n;
+    }
+    void reserve(int, hipStream_t s) const override { reserve_linear_scratch(s); }
+    void add_cost(StepCost& c) const override {
+        in_.add_cost(c);
+        out_.add_cost(c);
+        c.attention_flops_per_key += 2.0 * sh_.n_heads * (sh_.dim + sh_.value_dim);
+    }
+
+private:
+    ScoredShape sh_;
+    int dtype_ = BF16, k_col_ = 0, v_col_ = 0, gate_col_ = 0;
+    bool values_from_keys_ = false, gated_ = false;
+    Linear in_, out_;
+};
+
+}  // namespace
+
+void register_scored_attention() {
+    register_mixer("scored_attention", [](const Params& p) { return std::unique_ptr<Mixer>(new ScoredAttention(p)); });
+}
+
+}  // namespace minillm

@@ -276,6 +276,33 @@ DeviceTensors::~DeviceTensors() {
     for (void* p : ptrs_) (void)hipFree(p);
 }
 
+Tensor2 DeviceTensors::join_rows(const std::vector<Tensor2>& parts) {
+    if (parts.empty()) throw WeightsError("join_rows: nothing to join");
+    int64_t rows = 0;
+    for (const Tensor2& t : parts) {
+        if (t.dtype != parts[0].dtype || t.cols != parts[0].cols || !t.contiguous()) throw WeightsError("join_rows: the parts must be contiguous, of one dtype and width");
+        rows += t.rows;
+    }
+    const size_t row_bytes = static_cast<size_t>(parts[0].cols) * parts[0].esz();
+    char* base = static_cast<char*>(allocate(static_cast<size_t>(rows) * row_bytes, false));
+    size_t at = 0;
+    for (const Tensor2& t : parts) {
+        const size_t bytes = static_cast<size_t>(t.rows) * row_bytes;
+        if (bytes > 0 && hipMemcpy(base + at, t.data, bytes, hipMemcpyDeviceToDevice) != hipSuccess) throw WeightsError("join_rows: the copy on the device failed");
+        at += bytes;
+    }
+    return Tensor2(base, parts[0].dtype, rows, parts[0].cols);
+}
+
+Tensor2 DeviceTensors::repeat(const Tensor2& v, int times) {
+    if (v.dtype != F32 || !v.contiguous() || times < 1) throw WeightsError("repeat: a contiguous float32 vector and a positive count are needed");
+    const size_t n = static_cast<size_t>(v.rows) * v.cols;
+    char* base = static_cast<char*>(allocate(n * 4 * times, false));
+    for (int i = 0; i < times; ++i)
+        if (n > 0 && hipMemcpy(base + i * n * 4, v.data, n * 4, hipMemcpyDeviceToDevice) != hipSuccess) throw WeightsError("repeat: the copy on the device failed");
+    return Tensor2(base, F32, 1, static_cast<int64_t>(n) * times);
+}
+
 void* DeviceTensors::allocate(size_t bytes, bool zero) {
     void* p = nullptr;
     hipError_t e = hipMalloc(&p, std::max<size_t>(bytes, 16));
@@ -372,6 +399,8 @@ std::map<std::string, Tensor2> load_tensors(const std::vector<ParamSpec>& specs,
         if (s.shape.size() == 1) cols = s.shape[0];
         else if (s.shape.size() == 2) { rows = s.shape[0]; cols = s.shape[1]; }
         else throw WeightsError(where + ": tensor '" + s.name + "' has " + std::to_string(s.shape.size()) + " dimensions; one or two are expected");
+        if (s.add != 0.0)
+            for (auto& v : values) v = static_cast<float>(v + s.add);
         const std::vector<float>* src = &values;
         if (s.transpose) {
             turned.resize(values.size());

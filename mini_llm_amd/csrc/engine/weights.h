@@ -92,6 +92,7 @@ struct ParamSpec {
     enum Role { Matrix, Vector } role;   // matrix: kept in the compute dtype; vector: kept in fp32
     bool transpose = false;              // stored [in, out], used as [out, in]
     double mean = 0.0, std = 0.02;
+    double add = 0.0;                    // added to every value while loading (a weight stored around zero and used as 1 + w)
 };
 
 // Where tensors come from: a checkpoint on disk or the random generator. Gives fp32 host values.
@@ -145,6 +146,11 @@ public:
     // Uploads float32 host values [rows, cols] as `dtype` (bf16: round to nearest even) and returns the view.
     Tensor2 upload(const std::vector<float>& values, int64_t rows, int64_t cols, int dtype);
     void* allocate(size_t bytes, bool zero);
+    // Matrices of one width and dtype one below the other ([sum of rows, cols], a copy on the device): several
+    // linear maps of one input as one product.
+    Tensor2 join_rows(const std::vector<Tensor2>& parts);
+    // A vector `times` times in a row ([1, times * n] fp32, a copy on the device).
+    Tensor2 repeat(const Tensor2& vector, int times);
     size_t bytes() const { return bytes_; }
 
 private:

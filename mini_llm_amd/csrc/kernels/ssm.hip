@@ -41,6 +41,32 @@ __global__ void conv_silu_kernel(const float* __restrict__ proj, int ld, int col
     out[static_cast<size_t>(t) * ldo + ch] = silu_precise(acc);
 }
 
+// out[t, ch] = in[t, ch] + sum_j w[ch, j] * in(t - (taps - 1 - j), ch): the convolution added onto its own input,
+// no bias and no activation, the result in the activation dtype. Carried rows as above.
+template <typename OutT>
+__global__ void conv_residual_kernel(const float* __restrict__ in, int ld, int C, const float* __restrict__ w, int taps,
+                                     const int* __restrict__ token_seq, const int* __restrict__ cu_q,
+                                     const int* __restrict__ state_slots, float* __restrict__ state, size_t slot_floats,
+                                     OutT* __restrict__ out, int ldo, long long total, int carry) {
+    const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int t = static_cast<int>(i / C), ch = static_cast<int>(i % C);
+    const int b = token_seq[t], slot = state_slots[b];
+    if (slot < 0) return;
+    const int first = cu_q[b], k = t - first;
+    float* carried = state + static_cast<size_t>(slot) * slot_floats;
+    float acc = 0.f, own = 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int idx = k - (taps - 1 - j);
+        const float v = idx >= 0 ? in[static_cast<size_t>(first + idx) * ld + ch]
+                                 : carried[static_cast<size_t>(taps - 1 + idx) * C + ch];
+        acc += w[static_cast<size_t>(ch) * taps + j] * v;
+        own = v;
+        if (carry && j >= 1) carried[static_cast<size_t>(j - 1) * C + ch] = v;
+    }
+    out[static_cast<size_t>(t) * ldo + ch] = from_float<OutT>(own + acc);
+}
+
 // The slot's carried rows after the portion: its last taps - 1 inputs, older ones shifted out; a portion
 // shorter than that keeps the newest of the old rows. One thread per (sequence, channel); taps - 1 <= 15.
 __global__ void conv_carry_kernel(const float* __restrict__ proj, int ld, int col0, int C, int taps,
@@ -400,6 +426,32 @@ int mllm_conv_silu(const float* proj, int ld, int col0, int C, const float* w, c
     if (write && taps > 1 && !single) {
         const long long pairs = static_cast<long long>(B) * C;
         conv_carry_kernel<<<static_cast<int>((pairs + 255) / 256), 256, 0, stream>>>(proj, ld, col0, C, taps, cu_q, state_slots, state,
+                                                                                    slot_floats, B);
+        MLLM_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+// out = in + conv(in) over the C columns of in's rows (fp32), out in out_dtype; the slots' carried rows are brought
+// up to date as by mllm_conv_silu. -1: taps outside 1..16.
+int mllm_conv_residual(const float* in, int ld, int C, const float* w, int taps, const int* token_seq, const int* cu_q,
+                       const int* state_slots, float* state, size_t slot_floats, void* out, int ldo, int out_dtype, int T,
+                       int B, int write, hipStream_t stream) {
+    if (T <= 0 || C <= 0) return 0;
+    if (taps < 1 || taps > 16) return -1;
+    const long long total = static_cast<long long>(T) * C;
+    const bool single = T == B && write && taps > 1;
+    const int blocks = static_cast<int>((total + 255) / 256);
+    if (out_dtype == MLLM_F32)
+        conv_residual_kernel<float><<<blocks, 256, 0, stream>>>(in, ld, C, w, taps, token_seq, cu_q, state_slots, state, slot_floats,
+                                                                static_cast<float*>(out), ldo, total, single ? 1 : 0);
+    else
+        conv_residual_kernel<bf16_t><<<blocks, 256, 0, stream>>>(in, ld, C, w, taps, token_seq, cu_q, state_slots, state, slot_floats,
+                                                                 static_cast<bf16_t*>(out), ldo, total, single ? 1 : 0);
+    MLLM_LAUNCH_CHECK();
+    if (write && taps > 1 && !single) {
+        const long long pairs = static_cast<long long>(B) * C;
+        conv_carry_kernel<<<static_cast<int>((pairs + 255) / 256), 256, 0, stream>>>(in, ld, 0, C, taps, cu_q, state_slots, state,
                                                                                     slot_floats, B);
         MLLM_LAUNCH_CHECK();
     }
