@@ -44,7 +44,10 @@ void conv_residual(const Tensor2& in, const Tensor2& weight, const StateArgs& st
     const int C = i32(weight.rows), taps = i32(weight.cols);
     if (!weight.contiguous() || taps < 1 || taps > 16) fail("conv_residual: taps [channels, 1 to 16] contiguous are needed");
     if (in.cols != C || out.cols != C || out.rows != in.rows) fail("conv_residual: input and out must be [T, %d]", C);
-    check_state(st, static_cast<size_t>(taps - 1) * C, "conv_residual");
+    // (a single tap reads no carried rows: such a convolution needs no state, only the step's arrays)
+    if (taps > 1) check_state(st, static_cast<size_t>(taps - 1) * C, "conv_residual");
+    else if (st.token_seq == nullptr || st.cu_q == nullptr || st.state_slots == nullptr || st.n_seqs < 1)
+        fail("conv_residual: the step's token_seq, cu_q and state slots are needed");
     check(mllm_conv_residual(static_cast<const float*>(in.data), i32(in.stride), C, static_cast<const float*>(weight.data), taps, st.token_seq,
                              st.cu_q, st.state_slots, st.state, st.slot_floats, out.data, i32(out.stride), out.dtype, i32(in.rows), st.n_seqs,
                              st.write ? 1 : 0, stream), "conv_residual");

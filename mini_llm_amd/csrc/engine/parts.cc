@@ -330,7 +330,7 @@ public:
                  hipStream_t s) const override {
         size_t mark = arena.mark();
         if (conv_.data != nullptr) {
-            if (!cache.has_state() || cache.state_bytes < conv_bytes_) fail("a block with an input convolution needs %zu bytes of state per request", conv_bytes_);
+            if (conv_bytes_ > 0 && (!cache.has_state() || cache.state_bytes < conv_bytes_)) fail("a block with an input convolution needs %zu bytes of state per request", conv_bytes_);
             if (x.cols != conv_.rows) fail("the input convolution has %lld channels, the stream %lld", (long long)conv_.rows, (long long)x.cols);
             Tensor2 hn = arena.tensor(F32, x.rows, x.cols);      // the convolution reads the normed rows in fp32
             norm1_->forward_into(x, nullptr, hn, s);
@@ -342,9 +342,11 @@ public:
             conv_residual(hn, conv_, st, hc, s);
             StageTimes::get().mark("input_conv", s);
             CacheView rest = cache;                     // what lies behind the carried rows is the mixer's
-            rest.state = static_cast<char*>(cache.state) + conv_bytes_;
-            rest.state_bytes = cache.state_bytes - conv_bytes_;
-            if (rest.state_bytes == 0) rest.kind &= ~2;
+            if (conv_bytes_ > 0) {
+                rest.state = static_cast<char*>(cache.state) + conv_bytes_;
+                rest.state_bytes = cache.state_bytes - conv_bytes_;
+                if (rest.state_bytes == 0) rest.kind &= ~2;
+            }
             NormedInput h(hc);
             mixer_->forward(h, step, rest, x, write, arena, s);
         } else {
