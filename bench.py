@@ -61,6 +61,34 @@ def kugulorn_config(n_layer, size="gpt2-small", n_positions=1024):
             "vocab_size": 50257, "n_positions": n_positions, "n_layer": n}
 
 
+def rekirax_config(n_layer, size="gpt2-small", n_positions=1024):
+    """A Rekirax model that runs as many layers as the GPT-2 configuration `size` has, at the same width, vocabulary
+    and context: layers of chunked attention beside an HGRN2 recurrence (twice) and of windowed attention (once) in
+    turn, heads of 64 as many as GPT-2 has, a quarter as many key/value heads, windows and chunks of 512, 32 rotated
+    columns, four taps, each layer with a gated feed-forward whose three matrices hold what GPT-2's two do; the
+    layers 1 to 3 run twice (so the list is three layers shorter than the number of runs)."""
+    full_layers, d, h, f = SIZES[size]
+    runs = n_layer or full_layers
+    n = max(runs - 3, 4)
+    kv = max(k for k in range(1, max(h // 4, 1) + 1) if h % k == 0)
+    mlp = {"kind": "dense", "ff": f * 2 // 3 // 64 * 64}
+    layers = []
+    for i in range(n):
+        if i % 3 == 2:
+            layers.append({"type": "attention", "mlp": mlp,
+                           "mixer": {"heads": h, "kv_heads": kv, "dim": 64, "vdim": 64, "scale": 0.125, "softcap": 30.0, "mask": {"size": 512}}})
+        else:
+            left = {"heads": h, "kv_heads": kv, "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 512}, "rot": {"base": 10000.0, "dims": 32}}
+            layers.append({"type": "parallel", "mlp": mlp, "mixer": {"left": left, "right": {"heads": h, "dim": 64, "vdim": 64}}})
+    return {"architecture": "Rekirax", "vocab": 50257, "width": d, "norm": {"eps": 1e-6}, "canon": {"taps": 4},
+            "loop": {"start": 1, "stop": 4, "times": 2}, "layers": layers,
+            # (what the measurement itself reads; the architecture ignores them)
+            "vocab_size": 50257, "n_positions": n_positions, "n_layer": n + 3}
+
+
+DESIGNS = {"kugulorn": kugulorn_config, "rekirax": rekirax_config}
+
+
 def decode_run(model_dir, dtype, batch, prompt_len, steps, warmup, cfg):
     """Decode steps of `batch` requests through the whole engine. Every prompt is fed in ONE step before
     the clock starts, so that all requests decode in lockstep from position prompt_len on. Returns
@@ -238,11 +266,12 @@ def serving_main(args, cfg, model_dir):
 def compare_main(args):
     """--compare: both designs at one size through prefill_run and decode_run."""
     from mini_llm_amd import Runner, write_random_model
-    out = {"metric": f"Kugulorn beside GPT-2 at {args.size} sizes: prefill tok/s (2 x 1,024 tokens) and decode tok/s",
+    other = args.design if args.design in DESIGNS else "kugulorn"
+    out = {"metric": f"{other.capitalize()} beside GPT-2 at {args.size} sizes: prefill tok/s (2 x 1,024 tokens) and decode tok/s",
            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights seed 2, uniform random token ids)",
            "n_gpus": 1, "designs": {}}
-    for design in ("gpt2", "kugulorn"):
-        cfg = (kugulorn_config if design == "kugulorn" else small_config)(args.layers, args.size, args.positions)
+    for design in ("gpt2", other):
+        cfg = (DESIGNS[design] if design in DESIGNS else small_config)(args.layers, args.size, args.positions)
         with tempfile.TemporaryDirectory() as d:
             write_random_model(dict(cfg), d, seed=2)
             r = Runner(model_dir=d, dtype=args.dtype, page_size=16, n_pages=8, max_num_seqs=1)
@@ -258,8 +287,8 @@ def compare_main(args):
                 rec[f"decode_b{b}"] = {"tok_per_s": round(tps, 1), "ms_per_step": round(step_s * 1e3, 4), "mean_context": round(mean_ctx, 1),
                                        "GBps": round(bytes_step / step_s / 1e9, 1), "frac_of_hbm_peak": round(bytes_step / step_s / HBM_PEAK, 5)}
             out["designs"][design] = rec
-    g, k = out["designs"]["gpt2"], out["designs"]["kugulorn"]
-    out["kugulorn_over_gpt2"] = {"prefill": round(k["prefill"]["tok_per_s"] / g["prefill"]["tok_per_s"], 3),
+    g, k = out["designs"]["gpt2"], out["designs"][other]
+    out[other + "_over_gpt2"] = {"prefill": round(k["prefill"]["tok_per_s"] / g["prefill"]["tok_per_s"], 3),
                                  **{f"decode_b{b}": round(k[f"decode_b{b}"]["tok_per_s"] / g[f"decode_b{b}"]["tok_per_s"], 3) for b in (1, 8, 64)}}
     print(json.dumps(out))
     return 0
@@ -289,11 +318,11 @@ def main():
     ap.add_argument("--config", help="a config.json to measure in place of the GPT-2 sizes (any registered architecture; "
                                      "it names vocab_size and n_positions, or --vocab / --positions do)")
     ap.add_argument("--vocab", type=int, default=0, help="with --config: the vocabulary to draw token ids from")
-    ap.add_argument("--design", default="gpt2", choices=["gpt2", "kugulorn"],
-                    help="kugulorn: a Kugulorn model of about the size --size names (kugulorn_config) through the same "
-                         "measurement; --compare runs both designs one after the other")
+    ap.add_argument("--design", default="gpt2", choices=["gpt2", "kugulorn", "rekirax"],
+                    help="kugulorn / rekirax: a model of that design of about the size --size names (kugulorn_config, "
+                         "rekirax_config) through the same measurement; --compare runs it and GPT-2 one after the other")
     ap.add_argument("--compare", action="store_true",
-                    help="prefill (2 x 1,024 tokens) and decode (batch 1, 8, 64) of the Kugulorn model and of the GPT-2 model "
+                    help="prefill (2 x 1,024 tokens) and decode (batch 1, 8, 64) of the --design model (default Kugulorn) and of the GPT-2 model "
                          "of --size, side by side in one JSON line")
     ap.add_argument("--peaks-only", action="store_true",
                     help="measure this GPU's streaming bandwidth and matrix-core rate and print them")
@@ -311,8 +340,8 @@ def main():
     cfg = small_config(args.layers, args.size, args.positions)
     if args.compare:
         return compare_main(args)
-    if args.design == "kugulorn":
-        cfg = kugulorn_config(args.layers, args.size, args.positions)
+    if args.design in DESIGNS:
+        cfg = DESIGNS[args.design](args.layers, args.size, args.positions)
     if args.config:
         # another architecture, served by the same engine: sizes from its own config.json
         with open(args.config) as f:
@@ -366,7 +395,7 @@ def main():
             "higher_is_better": True, "scaling": "weak",
             "vs_baseline": round(tps / reference_tps, 2) if reference_tps else None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic (random weights seed 2, uniform random token ids)",
-            "config": {"model": args.size + "-sizes" + (" (Kugulorn)" if args.design == "kugulorn" else ""),
+            "config": {"model": args.size + "-sizes" + (f" ({args.design.capitalize()})" if args.design in DESIGNS else ""),
                        "n_layer": cfg["n_layer"], "n_layer_full": SIZES[args.size][0],
                        "n_embd": cfg.get("n_embd"), "n_head": cfg.get("n_head"),
                        "head_dim": cfg["n_embd"] // cfg["n_head"] if "n_embd" in cfg else None,

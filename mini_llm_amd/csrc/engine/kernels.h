@@ -115,7 +115,10 @@ int mllm_scored_attention_rows(const void* q, int ldq, const void* k_pages, cons
 int mllm_hgrn2_parts(int d);
 int mllm_hgrn2_scan(const float* proj, int ld, int q_col, int f_col, int v_col, const float* f_bias, const float* lower,
                     const int* cu_q, const int* state_slots, float* state, size_t slot_floats, size_t state_offset, float* y, int ldy,
-                    size_t part_stride, int T, int B, int H, int d, int dv, int write, hipStream_t stream);
+                    size_t part_stride, int T, int B, int max_q_len, int H, int d, int dv, int write, float* workspace,
+                    hipStream_t stream);
+size_t mllm_hgrn2_workspace_floats(int T, int B, int H, int d, int dv);
+int mllm_hgrn2_chunk();
 int mllm_concat_cast(const float* a, const float* b, int T, int D, void* out, int dtype, hipStream_t stream);
 int mllm_glu_act(const void* gu, int ld, int T, int F, int act, void* out, int ldo, int dtype, hipStream_t stream);
 

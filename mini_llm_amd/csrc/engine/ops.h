@@ -276,9 +276,14 @@ void scored_attention(const Tensor2& q, const Tensor2& k_pages, const Tensor2& v
 // proj (fp32 rows): raw queries at q_col and raw gates at f_col (heads * dim each), values at v_col (heads * value_dim).
 // y: hgrn2_parts(dim) shares [T, heads * value_dim], y.rows * y.stride floats apart; the state ([heads][dim][value_dim]
 // fp32) lies state_offset floats into a request's slot.
+// Portions longer than hgrn2_chunk() tokens are cut into chunks that run side by side, for which `workspace`
+// (hgrn2_workspace_floats floats) is needed; without it they run token by token.
 void hgrn2_scan(const Tensor2& proj, int q_col, int f_col, int v_col, const float* f_bias, const float* lower, const StateArgs& st,
-                size_t state_offset, int heads, int dim, int value_dim, const Tensor2& y, hipStream_t stream);
+                size_t state_offset, int heads, int dim, int value_dim, const Tensor2& y, float* workspace, size_t workspace_floats,
+                hipStream_t stream);
 int hgrn2_parts(int dim);
+int hgrn2_chunk();
+size_t hgrn2_workspace_floats(int tokens, int n_seqs, int heads, int dim, int value_dim);
 // out = [a | b] row by row in out's dtype (a, b fp32 [T, D])
 void concat_cast(const Tensor2& a, const Tensor2& b, const Tensor2& out, hipStream_t stream);
 // out[t, j] = act(gu[t, j]) * gu[t, F + j] (act: GELU_TANH)

@@ -106,9 +106,14 @@ void scored_attention(const Tensor2& q, const Tensor2& k_pages, const Tensor2& v
 }
 
 int hgrn2_parts(int dim) { return mllm_hgrn2_parts(dim); }
+int hgrn2_chunk() { return mllm_hgrn2_chunk(); }
+size_t hgrn2_workspace_floats(int tokens, int n_seqs, int heads, int dim, int value_dim) {
+    return mllm_hgrn2_workspace_floats(tokens, n_seqs, heads, dim, value_dim);
+}
 
 void hgrn2_scan(const Tensor2& proj, int q_col, int f_col, int v_col, const float* f_bias, const float* lower, const StateArgs& st,
-                size_t state_offset, int heads, int dim, int value_dim, const Tensor2& y, hipStream_t stream) {
+                size_t state_offset, int heads, int dim, int value_dim, const Tensor2& y, float* workspace, size_t workspace_floats,
+                hipStream_t stream) {
     need_f32(proj, "hgrn2_scan: the projection");
     need_f32(y, "hgrn2_scan: y");
     if (heads < 1 || dim < 1 || value_dim < 1) fail("hgrn2_scan: heads and sizes must be positive");
@@ -118,9 +123,14 @@ void hgrn2_scan(const Tensor2& proj, int q_col, int f_col, int v_col, const floa
     if (y.rows != proj.rows || y.cols != nv) fail("hgrn2_scan: y must be [%lld, %lld]", (long long)proj.rows, (long long)nv);
     if (lower == nullptr) fail("hgrn2_scan: the gates' lower bounds are needed");
     check_state(st, state_offset + static_cast<size_t>(heads) * dim * value_dim, "hgrn2_scan");
+    const int T = i32(proj.rows);
+    // (a step whose longest portion is unknown is taken to have a long one)
+    const int max_q = st.max_q_len > 0 ? st.max_q_len : T;
+    if (workspace != nullptr && workspace_floats < hgrn2_workspace_floats(T, st.n_seqs, heads, dim, value_dim))
+        fail("hgrn2_scan: the workspace holds %zu floats, %zu are needed", workspace_floats, hgrn2_workspace_floats(T, st.n_seqs, heads, dim, value_dim));
     check(mllm_hgrn2_scan(static_cast<const float*>(proj.data), i32(proj.stride), q_col, f_col, v_col, f_bias, lower, st.cu_q, st.state_slots,
                           st.state, st.slot_floats, state_offset, static_cast<float*>(y.data), i32(y.stride), static_cast<size_t>(y.rows) * y.stride,
-                          i32(proj.rows), st.n_seqs, heads, dim, value_dim, st.write ? 1 : 0, stream), "hgrn2_scan");
+                          T, st.n_seqs, max_q, heads, dim, value_dim, st.write ? 1 : 0, workspace, stream), "hgrn2_scan");
 }
 
 void concat_cast(const Tensor2& a, const Tensor2& b, const Tensor2& out, hipStream_t stream) {

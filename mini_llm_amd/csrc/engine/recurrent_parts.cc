@@ -50,7 +50,10 @@ public:
         // (the scan leaves its result as shares, one per slice of the key channels; the norm adds them)
         const int parts = hgrn2_parts(d_);
         Tensor2 y(arena.take(static_cast<size_t>(parts) * T * inner * 4), F32, T, inner);
-        hgrn2_scan(proj, 0, H_ * d_, 2 * H_ * d_, f_bias_, lower_, st, 0, H_, d_, dv_, y, s);
+        // (portions longer than a chunk are scanned chunk by chunk side by side: room for the chunks' states)
+        const size_t ws_floats = step.max_q_len > hgrn2_chunk() ? hgrn2_workspace_floats(T, step.n_seqs, H_, d_, dv_) : 0;
+        float* ws = ws_floats ? static_cast<float*>(arena.take(ws_floats * 4)) : nullptr;
+        hgrn2_scan(proj, 0, H_ * d_, 2 * H_ * d_, f_bias_, lower_, st, 0, H_, d_, dv_, y, ws, ws_floats, s);
         StageTimes::get().mark("scan", s);
         Tensor2 normed = arena.tensor(dtype_, T, inner);
         rmsnorm(y, norm_, eps_, H_, nullptr, normed, nullptr, s, parts, static_cast<size_t>(T) * inner);
@@ -58,7 +61,8 @@ public:
         StageTimes::get().mark("out_proj", s);
     }
     size_t workspace_bytes(int tokens) const override {
-        return static_cast<size_t>(tokens) * ((in_.out_features() + 4) * 4 + hgrn2_parts(d_) * H_ * dv_ * 4 + (H_ * dv_ + in_.in_features()) * dtype_size(dtype_)) + 4096;
+        return static_cast<size_t>(tokens) * ((in_.out_features() + 4) * 4 + hgrn2_parts(d_) * H_ * dv_ * 4 + (H_ * dv_ + in_.in_features()) * dtype_size(dtype_)) +
+               hgrn2_workspace_floats(tokens, 1, H_, d_, dv_) * 4 + 8192;
     }
     CacheNeed cache_need() const override {
         CacheNeed n;

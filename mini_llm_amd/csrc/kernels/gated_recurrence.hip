@@ -18,36 +18,74 @@ namespace {
 
 __device__ __forceinline__ float gr_sigmoid(float v) { return 1.f / (1.f + expf(-v)); }
 
+// MODE 0: every portion of the step is one chunk: from the slot's state, results to y, the state back to the slot.
+// Portions longer than GR_CHUNK tokens are cut into chunks that run side by side, in three launches:
+// MODE 1: every chunk from a zero state; it leaves its last state and the product of its gates in the workspace;
+//         then hgrn2_chunk_states_kernel walks a sequence's chunks in order, S <- F_c S + L_c, leaves in the
+//         workspace the state each chunk starts from, and writes the last state to the slot;
+// MODE 2: every chunk again, from the state it starts from, results to y.
+// The sums are those of the token-by-token recurrence in another order.
+// Workspace per chunk and head: [d * dv] the chunk's state, then [d] the product of its gates.
+#define GR_CHUNK 64
+
+template <int MODE>
 __global__ void __launch_bounds__(64)
 hgrn2_scan_kernel(const float* __restrict__ proj, int ld, int q_col, int f_col, int v_col, const float* __restrict__ f_bias,
                   const float* __restrict__ lower, const int* __restrict__ cu_q, const int* __restrict__ state_slots,
                   float* __restrict__ state, size_t slot_floats, float* __restrict__ y, int ldy, size_t part_stride, int H, int d,
-                  int dv, int n_tiles, int n_slices, int write) {
+                  int dv, int n_tiles, int n_slices, int write, int n_seqs, float* __restrict__ ws) {
     __shared__ float fq[2][2 * GR_ROWS];        // per token in turn: [f | q] of the slice's channels
     const int lane = threadIdx.x;
     int w = blockIdx.x;
     const int slice = w % n_slices; w /= n_slices;
     const int tile = w % n_tiles; w /= n_tiles;
-    const int h = w % H, b = w / H;
+    const int h = w % H;
+    w /= H;
+    int b, first, n, chunk_id = 0;
+    if (MODE == 0) {
+        b = w;
+        first = cu_q[b];
+        n = cu_q[b + 1] - first;
+    } else {
+        // which sequence and which of its chunks
+        chunk_id = w;
+        int c = w;
+        for (b = 0; b < n_seqs; ++b) {
+            first = cu_q[b];
+            n = cu_q[b + 1] - first;
+            const int nc = (n + GR_CHUNK - 1) / GR_CHUNK;
+            if (c < nc) break;
+            c -= nc;
+        }
+        if (b >= n_seqs) return;                // a surplus workgroup
+        first += c * GR_CHUNK;
+        n = min(GR_CHUNK, n - c * GR_CHUNK);
+    }
     const int slot = state_slots[b];
     if (slot < 0) return;
-    const int first = cu_q[b], n = cu_q[b + 1] - first;
     const int e = tile * 64 + lane, i0 = slice * GR_ROWS;
     const int rows = min(GR_ROWS, d - i0);
     const bool col_ok = e < dv;
     float* S = state + static_cast<size_t>(slot) * slot_floats + (static_cast<size_t>(h) * d + i0) * dv + (col_ok ? e : 0);
+    float* W = ws ? ws + (static_cast<size_t>(chunk_id) * H + h) * (static_cast<size_t>(d) * dv + d) : nullptr;
+    float* WS = W ? W + static_cast<size_t>(i0) * dv + (col_ok ? e : 0) : nullptr;
     float s[GR_ROWS];
 #pragma unroll
-    for (int i = 0; i < GR_ROWS; ++i) s[i] = (i < rows && col_ok) ? S[static_cast<size_t>(i) * dv] : 0.f;
+    for (int i = 0; i < GR_ROWS; ++i) {
+        s[i] = 0.f;
+        if (MODE == 0 && i < rows && col_ok) s[i] = S[static_cast<size_t>(i) * dv];
+        if (MODE == 2 && i < rows && col_ok) s[i] = WS[static_cast<size_t>(i) * dv];
+    }
     // the channel this lane prepares: lanes 0..31 the gate of channel lane, lanes 32..63 the query of channel lane - 32
     const int ch = lane % GR_ROWS;
     const bool ch_ok = ch < rows;
     const int c = h * d + i0 + (ch_ok ? ch : 0);
     const float lo = lower[c], fb = f_bias ? f_bias[c] : 0.f;
+    float cum = 1.f;                            // (lanes 0..31) the product of the channel's gates over the chunk
     for (int k = 0; k < n; ++k) {
         const float* row = proj + static_cast<size_t>(first + k) * ld;
         float val;
-        if (lane < GR_ROWS) val = lo + (1.f - lo) * gr_sigmoid(row[f_col + c] + fb);
+        if (lane < GR_ROWS) { val = lo + (1.f - lo) * gr_sigmoid(row[f_col + c] + fb); cum *= val; }
         else { const float z = row[q_col + c]; val = z * gr_sigmoid(z); }
         const float v = col_ok ? row[v_col + h * dv + e] : 0.f;
         float* cur = fq[k & 1];
@@ -60,13 +98,48 @@ hgrn2_scan_kernel(const float* __restrict__ proj, int ld, int q_col, int f_col, 
             s[i] = f * s[i] + (1.f - f) * v;
             o = fmaf(s[i], qi, o);
         }
-        if (col_ok) y[slice * part_stride + static_cast<size_t>(first + k) * ldy + h * dv + e] = o;
+        if (MODE != 1 && col_ok) y[slice * part_stride + static_cast<size_t>(first + k) * ldy + h * dv + e] = o;
     }
-    if (write && col_ok) {
+    if (MODE == 0 && write && col_ok) {
 #pragma unroll
         for (int i = 0; i < GR_ROWS; ++i)
             if (i < rows) S[static_cast<size_t>(i) * dv] = s[i];
     }
+    if (MODE == 1) {
+        if (col_ok) {
+#pragma unroll
+            for (int i = 0; i < GR_ROWS; ++i)
+                if (i < rows) WS[static_cast<size_t>(i) * dv] = s[i];
+        }
+        if (tile == 0 && lane < GR_ROWS && ch_ok) W[static_cast<size_t>(d) * dv + i0 + ch] = cum;
+    }
+}
+
+// One thread per (sequence, head, key channel, value column): the sequence's chunks in order. In the workspace a
+// chunk's own last state is replaced by the state it starts from.
+__global__ void hgrn2_chunk_states_kernel(const int* __restrict__ cu_q, const int* __restrict__ state_slots, float* __restrict__ state,
+                                          size_t slot_floats, float* __restrict__ ws, int H, int d, int dv, int n_seqs, int write) {
+    const long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const long long per_seq = static_cast<long long>(H) * d * dv;
+    if (idx >= per_seq * n_seqs) return;
+    const int b = static_cast<int>(idx / per_seq);
+    const long long r = idx % per_seq;
+    const int h = static_cast<int>(r / (static_cast<long long>(d) * dv)), i = static_cast<int>(r / dv % d);
+    const int slot = state_slots[b];
+    if (slot < 0) return;
+    int chunk0 = 0;
+    for (int bb = 0; bb < b; ++bb) chunk0 += (cu_q[bb + 1] - cu_q[bb] + GR_CHUNK - 1) / GR_CHUNK;
+    const int nc = (cu_q[b + 1] - cu_q[b] + GR_CHUNK - 1) / GR_CHUNK;
+    float* sp = state + static_cast<size_t>(slot) * slot_floats + r;
+    float S = *sp;
+    const size_t per_chunk = static_cast<size_t>(d) * dv + d;
+    for (int c = 0; c < nc; ++c) {
+        float* W = ws + (static_cast<size_t>(chunk0 + c) * H + h) * per_chunk;
+        const float L = W[r % (static_cast<long long>(d) * dv)], F = W[static_cast<size_t>(d) * dv + i];
+        W[r % (static_cast<long long>(d) * dv)] = S;
+        S = F * S + L;
+    }
+    if (write) *sp = S;
 }
 
 // out[t, :] = [a[t, :] | b[t, :]] in the output's dtype (two fp32 streams side by side, as one product's input)
@@ -101,18 +174,42 @@ int mllm_hgrn2_parts(int d) { return (d + GR_ROWS - 1) / GR_ROWS; }
 // request lies state_offset floats into its slot.
 int mllm_hgrn2_scan(const float* proj, int ld, int q_col, int f_col, int v_col, const float* f_bias, const float* lower,
                     const int* cu_q, const int* state_slots, float* state, size_t slot_floats, size_t state_offset, float* y, int ldy,
-                    size_t part_stride, int T, int B, int H, int d, int dv, int write, hipStream_t stream) {
+                    size_t part_stride, int T, int B, int max_q_len, int H, int d, int dv, int write, float* workspace,
+                    hipStream_t stream) {
     if (T <= 0 || B <= 0) return 0;
     if (H < 1 || d < 1 || dv < 1 || lower == nullptr) return -1;
     const int n_tiles = (dv + 63) / 64, n_slices = (d + GR_ROWS - 1) / GR_ROWS;
-    const long long blocks = static_cast<long long>(B) * H * n_tiles * n_slices;
-    if (blocks >= (1ll << 31)) return -1;
-    hgrn2_scan_kernel<<<static_cast<int>(blocks), 64, 0, stream>>>(proj, ld, q_col, f_col, v_col, f_bias, lower, cu_q, state_slots,
-                                                                  state + state_offset, slot_floats, y, ldy, part_stride, H, d, dv,
-                                                                  n_tiles, n_slices, write);
+    const long long per = static_cast<long long>(H) * n_tiles * n_slices;
+    if (max_q_len <= GR_CHUNK || workspace == nullptr) {
+        if (per * B >= (1ll << 31)) return -1;
+        hgrn2_scan_kernel<0><<<static_cast<int>(per * B), 64, 0, stream>>>(proj, ld, q_col, f_col, v_col, f_bias, lower, cu_q, state_slots,
+                                                                          state + state_offset, slot_floats, y, ldy, part_stride, H, d, dv,
+                                                                          n_tiles, n_slices, write, B, nullptr);
+        MLLM_LAUNCH_CHECK();
+        return 0;
+    }
+    const long long chunks = T / GR_CHUNK + B;          // an upper bound; surplus workgroups leave at once
+    if (per * chunks >= (1ll << 31)) return -1;
+    hgrn2_scan_kernel<1><<<static_cast<int>(per * chunks), 64, 0, stream>>>(proj, ld, q_col, f_col, v_col, f_bias, lower, cu_q, state_slots,
+                                                                           state + state_offset, slot_floats, y, ldy, part_stride, H, d, dv,
+                                                                           n_tiles, n_slices, write, B, workspace);
+    MLLM_LAUNCH_CHECK();
+    const long long cells = static_cast<long long>(B) * H * d * dv;
+    hgrn2_chunk_states_kernel<<<static_cast<int>((cells + 255) / 256), 256, 0, stream>>>(cu_q, state_slots, state + state_offset, slot_floats,
+                                                                                        workspace, H, d, dv, B, write);
+    MLLM_LAUNCH_CHECK();
+    hgrn2_scan_kernel<2><<<static_cast<int>(per * chunks), 64, 0, stream>>>(proj, ld, q_col, f_col, v_col, f_bias, lower, cu_q, state_slots,
+                                                                           state + state_offset, slot_floats, y, ldy, part_stride, H, d, dv,
+                                                                           n_tiles, n_slices, write, B, workspace);
     MLLM_LAUNCH_CHECK();
     return 0;
 }
+
+// Floats of workspace that a step of T tokens in B sequences needs when its longest portion exceeds a chunk.
+size_t mllm_hgrn2_workspace_floats(int T, int B, int H, int d, int dv) {
+    return static_cast<size_t>(T / GR_CHUNK + B) * H * (static_cast<size_t>(d) * dv + d);
+}
+int mllm_hgrn2_chunk() { return GR_CHUNK; }
 
 int mllm_concat_cast(const float* a, const float* b, int T, int D, void* out, int dtype, hipStream_t stream) {
     if (T <= 0 || D <= 0) return 0;
