@@ -57,20 +57,20 @@ LIBRARIES: Dict[str, dict] = {
     },
     # plain C++ twins of the device operations: the oracle of the kernel tests (host only)
     "ref": {"kind": "cxx", "sources": ["ref/ref_ops.cc"], "headers": []},
-    "elementwise": {"kind": "hip", "sources": ["kernels/elementwise.hip"], "headers": ["kernels/common.h"]},
-    "gemm_f32": {"kind": "hip", "sources": ["kernels/gemm_f32.hip"], "headers": ["kernels/common.h"]},
-    "gemm_bf16": {"kind": "hip", "sources": ["kernels/gemm_bf16.hip"], "headers": ["kernels/common.h"]},
-    "attention": {"kind": "hip", "sources": ["kernels/attention.hip"], "headers": ["kernels/common.h"]},
-    "attention_decode": {"kind": "hip", "sources": ["kernels/attention_decode.hip"], "headers": ["kernels/common.h"]},
-    "attention_prefill": {"kind": "hip", "sources": ["kernels/attention_prefill.hip"], "headers": ["kernels/common.h"]},
-    "norm_gate": {"kind": "hip", "sources": ["kernels/norm_gate.hip"], "headers": ["kernels/common.h"]},
-    "ssm": {"kind": "hip", "sources": ["kernels/ssm.hip"], "headers": ["kernels/common.h"]},
-    "latent_attention": {"kind": "hip", "sources": ["kernels/latent_attention.hip"], "headers": ["kernels/common.h"]},
-    "scored_attention": {"kind": "hip", "sources": ["kernels/scored_attention.hip"], "headers": ["kernels/common.h"]},
-    "gated_recurrence": {"kind": "hip", "sources": ["kernels/gated_recurrence.hip"], "headers": ["kernels/common.h"]},
+    "elementwise": {"kind": "hip", "sources": ["kernels/elementwise.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
+    "gemm_f32": {"kind": "hip", "sources": ["kernels/gemm_f32.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
+    "gemm_bf16": {"kind": "hip", "sources": ["kernels/gemm_bf16.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
+    "attention": {"kind": "hip", "sources": ["kernels/attention.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
+    "attention_decode": {"kind": "hip", "sources": ["kernels/attention_decode.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
+    "attention_prefill": {"kind": "hip", "sources": ["kernels/attention_prefill.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
+    "norm_gate": {"kind": "hip", "sources": ["kernels/norm_gate.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
+    "ssm": {"kind": "hip", "sources": ["kernels/ssm.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
+    "latent_attention": {"kind": "hip", "sources": ["kernels/latent_attention.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
+    "scored_attention": {"kind": "hip", "sources": ["kernels/scored_attention.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
+    "gated_recurrence": {"kind": "hip", "sources": ["kernels/gated_recurrence.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
     "sampling": {"kind": "hip", "sources": ["kernels/sampling.hip"],
-                 "headers": ["kernels/common.h", "kernels/noalloc.h"]},
-    "peaks": {"kind": "hip", "sources": ["kernels/peaks.hip"], "headers": ["kernels/common.h"]},
+                 "headers": ["kernels/common.h", "kernels/score_shape.h", "kernels/noalloc.h"]},
+    "peaks": {"kind": "hip", "sources": ["kernels/peaks.hip"], "headers": ["kernels/common.h", "kernels/score_shape.h"]},
     # the native engine: checked dispatch over the kernels, the parts, the model's step function
     # (host code only; it calls the kernel libraries' entry points)
     "engine": {
@@ -78,7 +78,7 @@ LIBRARIES: Dict[str, dict] = {
         "sources": ["engine/ops.cc", "engine/ops_sequence.cc", "engine/ops_scored.cc", "engine/parts.cc", "engine/parts_gated.cc",
                     "engine/mamba2.cc", "engine/latent_attention.cc", "engine/scored_attention.cc", "engine/recurrent_parts.cc", "engine/json.cc", "engine/weights.cc", "engine/arch.cc",
                     "engine/gpt2.cc", "engine/kugulorn.cc", "engine/rekirax.cc", "engine/engine.cc", "engine/engine_api.cc"],
-        "headers": ["engine/ops.h", "engine/parts.h", "engine/kernels.h", "engine/json.h", "engine/weights.h",
+        "headers": ["kernels/score_shape.h", "engine/ops.h", "engine/parts.h", "engine/kernels.h", "engine/json.h", "engine/weights.h",
                     "engine/arch.h", "engine/engine.h", "runtime/cache_manager.h", "runtime/scheduler.h"],
         "needs": ["elementwise", "gemm_f32", "gemm_bf16", "attention", "attention_decode", "attention_prefill",
                   "norm_gate", "ssm", "latent_attention", "scored_attention", "gated_recurrence", "sampling", "runtime"],

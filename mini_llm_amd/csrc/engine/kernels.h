@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 
+#include "score_shape.h"
+
 extern "C" {
 
 // elementwise.hip
@@ -47,20 +49,21 @@ int mllm_paged_attention_generic(const void* q, int q_stride, int q_col, const v
 int mllm_paged_attention_tiled(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
                                int kv_dim, const int* block_tables, int max_blocks, const int* cu_q, const int* ctx_len,
                                int n_seqs, int n_tiles_upper, int n_heads, int n_kv_heads, int head_dim, int page_size,
-                               float scale, int window, void* out, int out_stride, int dtype, hipStream_t stream);
+                               float scale, int window, void* out, int out_stride, int dtype, hipStream_t stream,
+                               const MllmScoreShape* shape = nullptr, const float* gate = nullptr, int ldg = 0);
 int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
                           int kv_dim, const int* block_tables, int max_blocks, const int* token_seq,
                           const int* positions, int n_q, int n_heads, int n_kv_heads, int head_dim,
                           int page_size, float scale, int window, int nsplit, int waves, void* out,
                           int out_stride, float* ws, int* counters, int k_col, int v_col, const int* slots,
-                          int partial_out, int dtype, hipStream_t stream);
+                          int partial_out, int dtype, hipStream_t stream, const MllmScoreShape* shape = nullptr);
 int mllm_merge_attention_splits(const float* ws, int n_q, int n_heads, int head_dim, int nsplit, void* out,
                                 int out_stride, int dtype, hipStream_t stream);
 int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
                                 int kv_dim, const int* block_tables, int max_blocks, const int* cu_q,
                                 const int* ctx_len, int n_seqs, int n_tiles_upper, int n_heads, int n_kv_heads,
                                 int head_dim, int page_size, float scale, int window, void* out, int out_stride,
-                                hipStream_t stream);
+                                hipStream_t stream, const MllmScoreShape* shape = nullptr, const float* gate = nullptr, int ldg = 0);
 
 // norm_gate.hip
 int mllm_rmsnorm(const float* x, int ldx, const int* rows, const float* w, const float* gate, int ldg, void* y, int ldy,
@@ -110,6 +113,8 @@ int mllm_scored_attention_rows(const void* q, int ldq, const void* k_pages, cons
                                int max_blocks, const int* token_seq, const int* positions, int n_tokens, int H, int G, int d,
                                int dv, int page_size, float scale, float softcap, int window, int chunk, const float* r1,
                                const float* r2, const float* gate, int ldg, void* out, int ldo, int dtype, hipStream_t stream);
+
+int mllm_gate_mul(void* x, int ldx, const float* gate, int ldg, int T, int N, int dtype, hipStream_t stream);
 
 // gated_recurrence.hip
 int mllm_hgrn2_parts(int d);

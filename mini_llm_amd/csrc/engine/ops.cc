@@ -389,6 +389,19 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
         fail("paged_attention: block tables, token_seq and positions are needed");
     if ((a.q.stride * esz) % 16 || (a.q_col * esz) % 16 || (a.head_dim * esz) % 16 || !aligned(a.q.data, 16))
         fail("paged_attention: query rows and heads must be 16-byte aligned");
+    if ((a.shape != nullptr || a.gate != nullptr) && (a.may_split || a.append))
+        fail("paged_attention: shaped scores and gates go with neither unmerged splits nor a fused append");
+    if (a.gate != nullptr && a.shape == nullptr) fail("paged_attention: a gate is taken with shaped scores only");
+    if (a.shape != nullptr && a.shape->chunk > 0 && a.window > 0) fail("paged_attention: a window or a chunk, not both");
+    // every row of a shaped attention through the kernel that takes any sizes
+    auto shaped_rows = [&](int n_rows) {
+        tuning().seen.generic_attention_launches += 1;
+        check(mllm_scored_attention_rows(a.q.data, static_cast<int>(a.q.stride), a.k_pages.data, a.v_pages.data, a.block_tables, a.max_blocks,
+                                         a.token_seq, a.positions, n_rows, a.n_heads, a.n_kv_heads, a.head_dim, a.head_dim, a.page_size,
+                                         a.scale, a.shape->softcap, a.window, a.shape->chunk, a.shape->r1, a.shape->r2, a.gate, a.gate_stride,
+                                         a.out.data, static_cast<int>(a.out.stride), a.q.dtype, stream), "scored_attention (rows)");
+    };
+    if (a.shape != nullptr && a.q_col != 0) fail("paged_attention: shaped scores take queries from column 0");
     const int lpk = a.head_dim * esz / 16;
     const bool single_ok = lpk >= 2 && pow2(lpk) && pow2(a.page_size) && a.max_blocks <= 4096;
     const bool decode = a.max_q_len == 1 && single_ok;
@@ -422,14 +435,14 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
                                               a.block_tables + static_cast<size_t>(first_seq) * a.max_blocks, a.max_blocks,
                                               a.cu_q + first_seq, a.ctx_len + first_seq, B, tiles, a.n_heads, a.n_kv_heads,
                                               a.head_dim, a.page_size, a.scale, a.window, a.out.data,
-                                              static_cast<int>(a.out.stride), stream), "prefill_attention");
+                                              static_cast<int>(a.out.stride), stream, a.shape, a.gate, a.gate_stride), "prefill_attention");
         } else {
             tuning().seen.tiled_f32_launches += 1;
             check(mllm_paged_attention_tiled(a.q.data, static_cast<int>(a.q.stride), a.q_col, a.k_pages.data, a.v_pages.data, kv_dim,
                                              a.block_tables + static_cast<size_t>(first_seq) * a.max_blocks, a.max_blocks,
                                              a.cu_q + first_seq, a.ctx_len + first_seq, B, tiles, a.n_heads, a.n_kv_heads,
                                              a.head_dim, a.page_size, a.scale, a.window, a.out.data,
-                                             static_cast<int>(a.out.stride), a.q.dtype, stream), "paged_attention (tiles)");
+                                             static_cast<int>(a.out.stride), a.q.dtype, stream, a.shape, a.gate, a.gate_stride), "paged_attention (tiles)");
         }
     };
     if ((tiles_ok || tiled_ok) && a.n_single > 0 && a.n_single < a.n_seqs) {
@@ -445,6 +458,8 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
             d.append = 0;
             d.may_split = 0;
             paged_attention(d, nullptr, stream);
+        } else if (a.shape != nullptr) {
+            shaped_rows(a.n_single);
         } else {
             tuning().seen.generic_attention_launches += 1;
             check(mllm_paged_attention_generic(a.q.data, static_cast<int>(a.q.stride), a.q_col, a.k_pages.data, a.v_pages.data, kv_dim,
@@ -471,12 +486,14 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
                                     a.block_tables, a.max_blocks, seq_of_token, a.positions, T, a.n_heads, a.n_kv_heads,
                                     a.head_dim, a.page_size, a.scale, a.window, nsplit, waves, a.out.data,
                                     static_cast<int>(a.out.stride), ws, counters, a.k_col, a.v_col, slots,
-                                    unmerged || merge_kernel ? 1 : 0, a.q.dtype, stream), "decode_attention");
+                                    unmerged || merge_kernel ? 1 : 0, a.q.dtype, stream, a.shape), "decode_attention");
         tuning().seen.max_decode_splits = std::max(tuning().seen.max_decode_splits, nsplit);
         if (merge_kernel) tuning().seen.merge_kernel_launches += 1;
         if (merge_kernel)
             check(mllm_merge_attention_splits(ws, T, a.n_heads, a.head_dim, nsplit, a.out.data, static_cast<int>(a.out.stride),
                                               a.q.dtype, stream), "merge_splits");
+        if (a.gate != nullptr)
+            check(mllm_gate_mul(a.out.data, static_cast<int>(a.out.stride), a.gate, a.gate_stride, T, q_dim, a.q.dtype, stream), "gate_mul");
         if (unmerged) {
             splits->ws = ws;
             splits->n_tokens = T;
@@ -492,6 +509,7 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
         portions(0);
         return false;
     }
+    if (a.shape != nullptr) { shaped_rows(T); return false; }
     tuning().seen.generic_attention_launches += 1;
     check(mllm_paged_attention_generic(a.q.data, static_cast<int>(a.q.stride), a.q_col, a.k_pages.data, a.v_pages.data, kv_dim,
                                        a.block_tables, a.max_blocks, a.token_seq, a.positions, T, a.n_heads, a.n_kv_heads,

@@ -15,6 +15,8 @@
 #include <stdexcept>
 #include <string>
 
+#include "score_shape.h"
+
 namespace minillm {
 
 enum DType : int { F32 = 0, BF16 = 1 };
@@ -84,6 +86,11 @@ struct AttentionArgs {
     const int* slots = nullptr;    // [T] rows of the pages (append)
     int n_single = 0;              // the first n_single sequences bring one token each
     int may_split = 0;             // != 0: the caller takes an AttentionSplits in place of `out`
+    // scores shaped before the softmax and a chunked mask (score_shape.h), or null; and a gate: the result is
+    // multiplied by sigmoid(gate[t, gate_col + column]) (fp32 rows, row stride gate_stride). Neither goes with may_split.
+    const MllmScoreShape* shape = nullptr;
+    const float* gate = nullptr;
+    int gate_stride = 0;
 };
 
 // -- scratch: device memory that kernels need beyond inputs and outputs, one set per stream -----------
@@ -107,6 +114,7 @@ struct Tuning {
     int long_context_splits = 1;                      // 1: few pairs with long contexts are split over up to 256 workgroups
     int ln_fuse_max_rows = 32;                        // rows up to which the norm is fused into the few-row product
     int latent_tiles = 1;                             // 1: latent attention's prompt portions may run on the matrix cores
+    int scored_shared_kernels = 1;                    // 1: attention with shaped scores may run on the kernels the plain attention runs on
     // what the ops chose since the last reset (tests read it back instead of trusting the thresholds)
     struct Seen {
         int max_decode_splits = 0;                    // most workgroups a (token, head) pair's keys were split over
@@ -262,6 +270,7 @@ void qk_prepare(const Tensor2& proj, int q_col, int k_col, int v_col, const Scor
 struct ScoredStep {
     const int* block_tables = nullptr;     // [n_seqs, max_blocks]
     int max_blocks = 0, n_seqs = 0, max_q_len = 0, max_ctx_len = 0, page_size = 0;
+    int n_single = 0;                      // the first n_single sequences bring one token each
     const int* token_seq = nullptr;        // [T]
     const int* positions = nullptr;        // [T]
     const int* cu_q = nullptr;             // [n_seqs + 1]

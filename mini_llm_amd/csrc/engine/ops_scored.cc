@@ -99,6 +99,23 @@ void scored_attention(const Tensor2& q, const Tensor2& k_pages, const Tensor2& v
         g = static_cast<const float*>(gate->data) + gate_col;
         ldg = i32(gate->stride);
     }
+    // keys and values of one width: the kernels that every attention of the engine runs on (tiles of queries for
+    // prompt portions, split keys for single tokens), with the shaping handed on; they fall back by themselves to
+    // the one-wavefront-per-row kernel below for sizes they do not take
+    if (tuning().scored_shared_kernels && sh.dim == sh.value_dim && sh.dim % 8 == 0 && sh.dim <= 256 && (q.stride * q.esz()) % 16 == 0 && (sh.dim * q.esz()) % 16 == 0 &&
+        (reinterpret_cast<uintptr_t>(q.data) & 15) == 0 && (g == nullptr || (ldg % 4 == 0 && (reinterpret_cast<uintptr_t>(g) & 15) == 0)) &&
+        step.cu_q != nullptr && step.ctx_len != nullptr && step.n_seqs > 0) {
+        const MllmScoreShape shape{sh.softcap, sh.chunk, sh.r1, sh.r2};
+        AttentionArgs a;
+        a.q = q; a.q_col = 0; a.n_heads = sh.n_heads; a.n_kv_heads = sh.n_kv_heads; a.head_dim = sh.dim;
+        a.k_pages = k_pages; a.v_pages = v_pages; a.page_size = step.page_size;
+        a.block_tables = step.block_tables; a.n_seqs = step.n_seqs; a.max_blocks = step.max_blocks;
+        a.token_seq = step.token_seq; a.positions = step.positions; a.scale = sh.scale; a.window = sh.window;
+        a.out = out; a.cu_q = step.cu_q; a.ctx_len = step.ctx_len; a.max_q_len = step.max_q_len; a.max_ctx_len = step.max_ctx_len;
+        a.n_single = step.n_single; a.shape = &shape; a.gate = g; a.gate_stride = ldg;
+        paged_attention(a, nullptr, stream);
+        return;
+    }
     check(mllm_scored_attention_rows(q.data, i32(q.stride), k_pages.data, v_pages.data, step.block_tables, step.max_blocks, step.token_seq,
                                      step.positions, i32(q.rows), sh.n_heads, sh.n_kv_heads, sh.dim, sh.value_dim, step.page_size, sh.scale,
                                      sh.softcap, sh.window, sh.chunk, sh.r1, sh.r2, g, ldg, out.data, i32(out.stride), q.dtype, stream),

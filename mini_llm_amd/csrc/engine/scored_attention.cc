@@ -75,7 +75,7 @@ public:
         ScoredStep st;
         st.block_tables = step.block_tables[g]; st.max_blocks = step.max_blocks[g]; st.n_seqs = step.n_seqs; st.max_q_len = step.max_q_len;
         st.max_ctx_len = step.max_ctx_len; st.page_size = cache.page_size; st.token_seq = step.token_seq; st.positions = step.positions;
-        st.cu_q = step.cu_q; st.ctx_len = step.ctx_len;
+        st.cu_q = step.cu_q; st.ctx_len = step.ctx_len; st.n_single = step.n_single;
         Tensor2 o = arena.tensor(dtype_, T, sh_.n_heads * sh_.value_dim);
         scored_attention(q, cache.k_pages, cache.v_pages, st, sh_, gated_ ? &proj : nullptr, gate_col_, o, s);
         StageTimes::get().mark("attention", s);
@@ -91,7 +91,10 @@ public:
         n.kind = 1; n.n_kv_heads = sh_.n_kv_heads; n.head_dim = sh_.dim; n.value_dim = sh_.value_dim; n.window = sh_.window;
         return n;
     }
-    void reserve(int, hipStream_t s) const override { reserve_linear_scratch(s); }
+    void reserve(int max_seqs, hipStream_t s) const override {
+        reserve_attention_scratch((max_seqs + 7) / 8 * 8, sh_.n_heads, sh_.dim, s);
+        reserve_linear_scratch(s);
+    }
     void add_cost(StepCost& c) const override {
         in_.add_cost(c);
         out_.add_cost(c);

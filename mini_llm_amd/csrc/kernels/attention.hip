@@ -137,13 +137,15 @@ template <> __device__ __forceinline__ void store4f<bf16_t>(bf16_t* p, f32x4_t v
 
 // DC: the most 16-dim chunks of a head (head_dim <= 16 DC); loops over chunks are unrolled to DC and
 // predicated, so that the register arrays are indexed by constants.
-template <typename T, int DC>
+// SHAPED: the scores are shaped before the softmax (score_shape.h), a chunked mask may stand in for the window, and
+// the result may be multiplied by the sigmoid of a gate (fp32 rows). The queries then come times the scale alone.
+template <typename T, int DC, bool SHAPED = false>
 __global__ void __launch_bounds__(256)
 paged_attention_tiled(const T* __restrict__ q, int q_stride, int q_col, const T* __restrict__ k_pages,
                       const T* __restrict__ v_pages, int kv_dim, const int* __restrict__ block_tables, int max_blocks,
                       const int* __restrict__ cu_q, const int* __restrict__ ctx_len, int n_seqs, int n_heads,
                       int n_kv_heads, int head_dim, int page_size, float scale_log2e, int window,
-                      T* __restrict__ out, int out_stride) {
+                      T* __restrict__ out, int out_stride, MllmScoreShape shape, const float* __restrict__ gate, int ldg) {
     extern __shared__ __attribute__((aligned(16))) float tl_smem[];
     const int n_c = head_dim / 16;                 // 16-dim chunks
     const int ldk = head_dim + 4;                  // floats per key row: (head_dim / 4 + 1) x 16 bytes, odd
@@ -170,8 +172,10 @@ paged_attention_tiled(const T* __restrict__ q, int q_stride, int q_col, const T*
     const bool q_ok = qi < q_len;
     const int p = start + min(qi, q_len - 1);      // its position (a lane beyond the last query repeats it; never stored)
     const int p_first = start + q0, p_last = start + min(q0 + TL_BQ, q_len) - 1;
-    const int k_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
-    const int my_lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    int k_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+    int my_lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    if (SHAPED && shape.chunk > 0) { k_lo = p_first - p_first % shape.chunk; my_lo = p - p % shape.chunk; }
+    const float r1 = (SHAPED && shape.r1) ? shape.r1[blockIdx.x] : 0.f, r2 = (SHAPED && shape.r1) ? shape.r2[blockIdx.x] : 0.f;
     // the last position any of this wavefront's queries may see (uniform over the wavefront)
     const int wave_last = start + min(q0 + wave * 16 + 15, q_len - 1);
     const int* table = block_tables + static_cast<size_t>(b) * max_blocks;
@@ -233,6 +237,7 @@ paged_attention_tiled(const T* __restrict__ q, int q_stride, int q_col, const T*
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int j = k0 + 16 * g + 4 * G + i;
+                if (SHAPED) s[g][i] = mllm_shaped_score(s[g][i], shape, r1, r2, max(p - j, 0)) * MLLM_LOG2E;
                 s[g][i] = (j <= p && j >= my_lo) ? s[g][i] : -INFINITY;
                 mx = fmaxf(mx, s[g][i]);
             }
@@ -268,8 +273,17 @@ paged_attention_tiled(const T* __restrict__ q, int q_stride, int q_col, const T*
     const float inv_l = 1.f / l;
     T* op = out + static_cast<size_t>(q_begin + qi) * out_stride + h * head_dim + 4 * G;
 #pragma unroll
-    for (int c = 0; c < DC; ++c)
-        if (c < n_c) store4f<T>(op + 16 * c, o[c] * inv_l);
+    for (int c = 0; c < DC; ++c) {
+        if (c < n_c) {
+            f32x4_t r = o[c] * inv_l;
+            if (SHAPED && gate != nullptr) {
+                const float* gp = gate + static_cast<size_t>(q_begin + qi) * ldg + h * head_dim + 4 * G + 16 * c;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) r[i] *= 1.f / (1.f + expf(-gp[i]));
+            }
+            store4f<T>(op + 16 * c, r);
+        }
+    }
 }
 
 extern "C" {
@@ -306,8 +320,11 @@ int mllm_paged_attention_generic(const void* q, int q_stride, int q_col, const v
 int mllm_paged_attention_tiled(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
                                int kv_dim, const int* block_tables, int max_blocks, const int* cu_q, const int* ctx_len,
                                int n_seqs, int n_tiles_upper, int n_heads, int n_kv_heads, int head_dim, int page_size,
-                               float scale, int window, void* out, int out_stride, int dtype, hipStream_t stream) {
+                               float scale, int window, void* out, int out_stride, int dtype, hipStream_t stream,
+                               const MllmScoreShape* shape, const float* gate, int ldg) {
     if (n_seqs <= 0 || n_tiles_upper <= 0) return 0;
+    if ((shape == nullptr && gate != nullptr) || (shape && window > 0 && shape->chunk > 0)) return -1;
+    const MllmScoreShape sh = shape ? *shape : MllmScoreShape{0.f, 0, nullptr, nullptr};
     if (head_dim % 16 != 0 || head_dim < 16 || head_dim > 256 || n_heads % n_kv_heads != 0 || n_tiles_upper > 65535 ||
         page_size < 1)
         return -1;
@@ -315,21 +332,28 @@ int mllm_paged_attention_tiled(const void* q, int q_stride, int q_col, const voi
     if ((q_stride * esz) % 16 || (q_col * esz) % 16 || (kv_dim * esz) % 16 || (out_stride * esz) % 8) return -1;
     const dim3 grid(n_heads, n_tiles_upper);
     const size_t smem = (static_cast<size_t>(TL_BK) * (head_dim + 4) + static_cast<size_t>(head_dim) * TL_VSTRIDE) * sizeof(float);
-    const float sl2 = scale * 1.44269504088896340736f;
+    const float sl2 = shape ? scale : scale * 1.44269504088896340736f;
 #define TL_CASE(TYPE, DC)                                                                                          \
     do {                                                                                                           \
         static bool lds_allowed = false;      /* more than 64 KB of LDS is asked for once */                       \
         if (!lds_allowed) {                                                                                        \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(paged_attention_tiled<TYPE, DC>),      \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(paged_attention_tiled<TYPE, DC, false>), \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize,                         \
+                                               static_cast<int>((TL_BK * (16 * DC + 4) + 16 * DC * TL_VSTRIDE) * sizeof(float))); \
+            if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(paged_attention_tiled<TYPE, DC, true>), \
                                                hipFuncAttributeMaxDynamicSharedMemorySize,                         \
                                                static_cast<int>((TL_BK * (16 * DC + 4) + 16 * DC * TL_VSTRIDE) * sizeof(float))); \
             if (e != hipSuccess) return static_cast<int>(e);                                                       \
             lds_allowed = true;                                                                                    \
         }                                                                                                          \
-        paged_attention_tiled<TYPE, DC><<<grid, 256, smem, stream>>>(                                              \
+        if (shape) paged_attention_tiled<TYPE, DC, true><<<grid, 256, smem, stream>>>(                             \
             (const TYPE*)q, q_stride, q_col, (const TYPE*)k_pages, (const TYPE*)v_pages, kv_dim, block_tables,     \
             max_blocks, cu_q, ctx_len, n_seqs, n_heads, n_kv_heads, head_dim, page_size, sl2, window, (TYPE*)out,   \
-            out_stride);                                                                                           \
+            out_stride, sh, gate, ldg);                                                                            \
+        else paged_attention_tiled<TYPE, DC, false><<<grid, 256, smem, stream>>>(                                  \
+            (const TYPE*)q, q_stride, q_col, (const TYPE*)k_pages, (const TYPE*)v_pages, kv_dim, block_tables,     \
+            max_blocks, cu_q, ctx_len, n_seqs, n_heads, n_kv_heads, head_dim, page_size, sl2, window, (TYPE*)out,   \
+            out_stride, sh, nullptr, 0);                                                                           \
     } while (0)
     const int dc = head_dim <= 64 ? 4 : head_dim <= 128 ? 8 : 16;
     if (dtype == MLLM_F32) {

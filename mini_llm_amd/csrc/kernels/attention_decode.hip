@@ -62,7 +62,9 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float (&o)[N], f
     m = mn;
 }
 
-template <typename T, int LPK, int UNR>
+// SHAPED: the scores are shaped before the softmax and a chunked mask may stand in for the window (score_shape.h);
+// the queries then come times the scale alone, and the shaped score goes to base 2 afterwards.
+template <typename T, int LPK, int UNR, bool SHAPED = false>
 __global__ void __launch_bounds__(UNR > 8 ? 512 : DEC_MAX_WAVES * MLLM_WAVE)
 decode_attention_kernel(// the first 16 dwords arrive in registers with the wavefront: what the first loads need
                         const int* __restrict__ token_seq, const int* __restrict__ positions,
@@ -73,7 +75,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
                         float scale_log2e, T* __restrict__ out, int out_stride,
                         float* __restrict__ ws_o, float* __restrict__ ws_ml, int* __restrict__ counters,
                         T* __restrict__ k_pages_w, T* __restrict__ v_pages_w, int k_col, int v_col,
-                        const int* __restrict__ slots, int partial_out) {
+                        const int* __restrict__ slots, int partial_out, MllmScoreShape shape) {
     constexpr int EPL = Vec16<T>::N;        // elements per lane
     constexpr int DH = LPK * EPL;           // head size
     constexpr int KPW = MLLM_WAVE / LPK;    // keys per wavefront and load instruction
@@ -99,7 +101,9 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
     if (whole_row)
         for (int i = threadIdx.x; i < max_blocks; i += blockDim.x) sm_table[i] = gtable_row[i];
     const int p = positions[t];
-    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    if (SHAPED && shape.chunk > 0) lo = p - p % shape.chunk;
+    const float r1 = (SHAPED && shape.r1) ? shape.r1[h] : 0.f, r2 = (SHAPED && shape.r1) ? shape.r2[h] : 0.f;
     const int n_keys = p - lo + 1;
     const int per = (n_keys + nsplit - 1) / nsplit;
     const int kb = lo + split * per;
@@ -174,6 +178,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
             for (int e = 0; e < EPL; ++e) d = fmaf(qf[e], kf[e], d);
             d = group_sum<LPK>(d);
             const bool valid = j0 + u * group_keys + g < ke_pages;
+            if (SHAPED) d = mllm_shaped_score(d, shape, r1, r2, valid ? p - (j0 + u * group_keys + g) : 0) * MLLM_LOG2E;
             dot[u] = valid ? d : NEG;
             mx = fmaxf(mx, dot[u]);
         }
@@ -202,6 +207,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
 #pragma unroll
         for (int e = 0; e < EPL; ++e) d = fmaf(qf[e], kf[e], d);
         d = group_sum<LPK>(d);
+        if (SHAPED) d = mllm_shaped_score(d, shape, r1, r2, 0) * MLLM_LOG2E;
         const float mn = fmaxf(m, d);
         const float a = exp2_for<T>(m - mn), pj = exp2_for<T>(d - mn);
         l = l * a + pj;
@@ -321,13 +327,15 @@ static int launch_decode(int lpk, dim3 grid, int waves, hipStream_t stream, cons
                          int max_blocks, const int* token_seq, const int* positions, int n_heads,
                          int n_kv_heads, int page_size, float scale_log2e, int window, int nsplit, T* out,
                          int out_stride, float* ws_o, float* ws_ml, int* counters, T* k_pages_w, T* v_pages_w,
-                         int k_col, int v_col, const int* slots, int partial_out) {
+                         int k_col, int v_col, const int* slots, int partial_out, const MllmScoreShape* shape) {
+    const MllmScoreShape sh = shape ? *shape : MllmScoreShape{0.f, 0, nullptr, nullptr};
 #define DEC_ARGS token_seq, positions, block_tables, max_blocks, n_heads, n_kv_heads, page_size, window,  \
             nsplit, q, q_stride, q_col, k_pages, v_pages, kv_dim, scale_log2e, out, out_stride,        \
-            ws_o, ws_ml, counters, k_pages_w, v_pages_w, k_col, v_col, slots, partial_out
+            ws_o, ws_ml, counters, k_pages_w, v_pages_w, k_col, v_col, slots, partial_out, sh
 #define DEC_CASE(L)                                                                                    \
     case L:                                                                                            \
-        decode_attention_kernel<T, L, 8><<<grid, waves * MLLM_WAVE, 0, stream>>>(DEC_ARGS);             \
+        if (shape) decode_attention_kernel<T, L, 8, true><<<grid, waves * MLLM_WAVE, 0, stream>>>(DEC_ARGS); \
+        else decode_attention_kernel<T, L, 8, false><<<grid, waves * MLLM_WAVE, 0, stream>>>(DEC_ARGS);  \
         return 0;
     switch (lpk) {
         DEC_CASE(2) DEC_CASE(4) DEC_CASE(8) DEC_CASE(16) DEC_CASE(32) DEC_CASE(64)
@@ -401,7 +409,7 @@ int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_
                           const int* positions, int n_q, int n_heads, int n_kv_heads, int head_dim,
                           int page_size, float scale, int window, int nsplit, int waves, void* out,
                           int out_stride, float* ws, int* counters, int k_col, int v_col, const int* slots,
-                          int partial_out, int dtype, hipStream_t stream) {
+                          int partial_out, int dtype, hipStream_t stream, const MllmScoreShape* shape) {
     if (n_q <= 0) return 0;
     const int esz = dtype == MLLM_F32 ? 4 : 2;
     const int lpk = head_dim * esz / 16;
@@ -411,18 +419,20 @@ int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_
     dim3 grid(n_q * n_heads, nsplit);
     float* ws_o = ws;
     float* ws_ml = ws + static_cast<size_t>(n_q) * n_heads * nsplit * head_dim;
-    const float sl2 = scale * 1.44269504088896340736f;
+    // (shaped scores: the queries times the scale alone; the kernel goes to base 2 after the shaping)
+    const float sl2 = shape ? scale : scale * 1.44269504088896340736f;
+    if (shape && window > 0 && shape->chunk > 0) return -1;
     int rc;
     if (dtype == MLLM_F32)
         rc = launch_decode<float>(lpk, grid, waves, stream, (const float*)q, q_stride, q_col, (const float*)k_pages,
                                   (const float*)v_pages, kv_dim, block_tables, max_blocks, token_seq, positions,
                                   n_heads, n_kv_heads, page_size, sl2, window, nsplit, (float*)out, out_stride,
-                                  ws_o, ws_ml, counters, (float*)k_pages, (float*)v_pages, k_col, v_col, slots, partial_out);
+                                  ws_o, ws_ml, counters, (float*)k_pages, (float*)v_pages, k_col, v_col, slots, partial_out, shape);
     else
         rc = launch_decode<bf16_t>(lpk, grid, waves, stream, (const bf16_t*)q, q_stride, q_col, (const bf16_t*)k_pages,
                                    (const bf16_t*)v_pages, kv_dim, block_tables, max_blocks, token_seq, positions,
                                    n_heads, n_kv_heads, page_size, sl2, window, nsplit, (bf16_t*)out, out_stride,
-                                   ws_o, ws_ml, counters, (bf16_t*)k_pages, (bf16_t*)v_pages, k_col, v_col, slots, partial_out);
+                                   ws_o, ws_ml, counters, (bf16_t*)k_pages, (bf16_t*)v_pages, k_col, v_col, slots, partial_out, shape);
     if (rc != 0) return rc;
     MLLM_LAUNCH_CHECK();
     return 0;

@@ -40,14 +40,17 @@ union Frag8 {
 
 // (At most 2 wavefronts per SIMD: the compiler may then use 256 registers, and keeps both
 // prefetched tiles in registers instead of private memory.)
-template <int DH, int NW>
+// SHAPED: the scores are shaped before the softmax (score_shape.h: cap, distance bias), a chunked mask may stand in
+// for the window, and the result may be multiplied by the sigmoid of a gate (fp32 rows, one value per output column).
+template <int DH, int NW, bool SHAPED = false>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, (DH >= 128 && NW == 4) ? 1 : 2)))
 prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages, int kv_dim,
                          const int* __restrict__ block_tables, int max_blocks,
                          const int* __restrict__ cu_q, const int* __restrict__ ctx_len, int n_seqs,
                          int n_heads, int n_kv_heads, int page_size, float scale_log2e, int window,
-                         bf16_t* __restrict__ out, int out_stride) {
+                         bf16_t* __restrict__ out, int out_stride, MllmScoreShape shape, float scale,
+                         const float* __restrict__ gate, int ldg) {
     constexpr int KS = DH / 32;            // k steps of S^T
     constexpr int DT = DH / 16;            // 16-dim tiles of O^T
     constexpr int KSTRIDE = DH + 8;
@@ -86,7 +89,12 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     const int p = start + qi;                             // its position
     const int p_first = start + q0;
     const int p_last = start + min(q0 + PF_BM, q_len) - 1;
-    const int k_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+    int k_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+    const int chunk = SHAPED ? shape.chunk : 0;
+    if (chunk > 0) k_lo = p_first - p_first % chunk;
+    const float r1 = (SHAPED && shape.r1) ? shape.r1[blockIdx.x] : 0.f, r2 = (SHAPED && shape.r1) ? shape.r2[blockIdx.x] : 0.f;
+    // (shaped scores are in base 2 already when they meet the exponent)
+    const float sl = SHAPED ? 1.f : scale_log2e;
     // The sequence's block table goes to LDS first: the gathers below then depend on an LDS read,
     // not on a global load that would have to be waited for in front of every key load.
     // (The host passes page sizes that are powers of two and tables of at most PF_TABLE_LDS blocks.)
@@ -182,9 +190,10 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 s[nt][r] = acc[r];                   // raw dot product; the scale is applied with the exponent
+                const int j = j_base + 16 * (nt0 + nt) + 4 * G + r;
+                if (SHAPED) s[nt][r] = mllm_shaped_score(acc[r] * scale, shape, r1, r2, max(p - j, 0)) * MLLM_LOG2E;
                 if (MASKED) {
-                    const int j = j_base + 16 * (nt0 + nt) + 4 * G + r;
-                    const bool seen = q_ok && j <= p && (window <= 0 || j > p - window);
+                    const bool seen = q_ok && j <= p && (window <= 0 || j > p - window) && (chunk <= 0 || j >= p - p % chunk);
                     if (!seen) s[nt][r] = -INFINITY;
                 }
                 tile_max = fmaxf(tile_max, s[nt][r]);
@@ -192,7 +201,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         }
         // the four lane groups of a query agree on the maximum
         tile_max = rows_max(tile_max);
-        const float m_new = fmaxf(m, tile_max * scale_log2e);        // the scale is positive
+        const float m_new = fmaxf(m, tile_max * sl);        // the scale is positive
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;      // nothing seen yet: all weights are 0
         const float alpha = fast_exp2(m - m_use);
         m = m_new;
@@ -201,7 +210,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         for (int nt = 0; nt < NT_PER; ++nt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                s[nt][r] = fast_exp2(fmaf(s[nt][r], scale_log2e, -m_use));
+                s[nt][r] = fast_exp2(fmaf(s[nt][r], sl, -m_use));
                 psum += s[nt][r];
             }
         l = l * alpha + psum;                 // this lane's share of the sum; merged over groups at the end
@@ -235,7 +244,8 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
 
     auto run_tile = [&](int kt, int buf) {
         const int j_base = kt * PF_BN;
-        const bool full = j_base + PF_BN - 1 <= pw_min && (window <= 0 || j_base > pw_max - window);
+        const bool full = j_base + PF_BN - 1 <= pw_min && (window <= 0 || j_base > pw_max - window) &&
+                          (chunk <= 0 || j_base >= pw_max - pw_max % chunk);
         if (full) compute(kt, buf, std::false_type{}); else compute(kt, buf, std::true_type{});
     };
 
@@ -312,9 +322,15 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     bf16_t* orow = out + static_cast<size_t>(q_begin + qi) * out_stride + h * DH;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
+        float g4[4] = {1.f, 1.f, 1.f, 1.f};
+        if (SHAPED && gate != nullptr) {
+            const float4 gv = *reinterpret_cast<const float4*>(gate + static_cast<size_t>(q_begin + qi) * ldg + blockIdx.x * DH + 16 * dt + 4 * G);
+            g4[0] = 1.f / (1.f + __expf(-gv.x)); g4[1] = 1.f / (1.f + __expf(-gv.y));
+            g4[2] = 1.f / (1.f + __expf(-gv.z)); g4[3] = 1.f / (1.f + __expf(-gv.w));
+        }
         uint2 pk;
-        pk.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
-        pk.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
+        pk.x = pack_bf16x2(o[dt][0] * inv * g4[0], o[dt][1] * inv * g4[1]);
+        pk.y = pack_bf16x2(o[dt][2] * inv * g4[2], o[dt][3] * inv * g4[3]);
         *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * G) = pk;
     }
 }
@@ -330,27 +346,36 @@ int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const vo
                                 int kv_dim, const int* block_tables, int max_blocks, const int* cu_q,
                                 const int* ctx_len, int n_seqs, int n_tiles_upper, int n_heads, int n_kv_heads,
                                 int head_dim, int page_size, float scale, int window, void* out, int out_stride,
-                                hipStream_t stream) {
+                                hipStream_t stream, const MllmScoreShape* shape, const float* gate, int ldg) {
     if (n_seqs <= 0 || n_tiles_upper <= 0) return 0;
+    // (the gate is read 16 bytes at a time)
+    if (shape == nullptr && gate != nullptr) return -1;
+    if (gate != nullptr && (ldg % 4 != 0 || (reinterpret_cast<uintptr_t>(gate) & 15) != 0)) return -1;
+    if (shape && window > 0 && shape->chunk > 0) return -1;
+    const MllmScoreShape sh = shape ? *shape : MllmScoreShape{0.f, 0, nullptr, nullptr};
     if (n_heads % n_kv_heads != 0 || n_tiles_upper > 65535) return -1;
     if ((page_size & (page_size - 1)) != 0 || page_size < head_dim / 16 || max_blocks > PF_TABLE_LDS) return -1;
     const dim3 grid(n_heads, n_tiles_upper);
     const size_t table_bytes = static_cast<size_t>(max_blocks) * sizeof(int);
     const float sl2 = scale * 1.44269504088896340736f;
-#define PF_CASE(D, W, KEY)                                                                                  \
-    case KEY: {                                                                                               \
+#define PF_LAUNCH(D, W, S)                                                                                  \
+    do {                                                                                                    \
         static bool lds_allowed = false;      /* static and dynamic LDS together pass 64 KB: asked for once */ \
         if (!lds_allowed) {                                                                                 \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_attention_kernel<D, W>), \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_attention_kernel<D, W, S>), \
                                                hipFuncAttributeMaxDynamicSharedMemorySize,                  \
                                                PF_TABLE_LDS * static_cast<int>(sizeof(int)));               \
             if (e != hipSuccess) return static_cast<int>(e);                                                \
             lds_allowed = true;                                                                             \
         }                                                                                                   \
-        prefill_attention_kernel<D, W><<<grid, W * 64, table_bytes, stream>>>(                                            \
+        prefill_attention_kernel<D, W, S><<<grid, W * 64, table_bytes, stream>>>(                           \
             (const bf16_t*)q, q_stride, q_col, (const bf16_t*)k_pages, (const bf16_t*)v_pages, kv_dim,      \
             block_tables, max_blocks, cu_q, ctx_len, n_seqs, n_heads, n_kv_heads, page_size, sl2, window,   \
-            (bf16_t*)out, out_stride);                                                                      \
+            (bf16_t*)out, out_stride, sh, scale, gate, ldg);                                                \
+    } while (0)
+#define PF_CASE(D, W, KEY)                                                                                  \
+    case KEY: {                                                                                             \
+        if (shape) PF_LAUNCH(D, W, true); else PF_LAUNCH(D, W, false);                                      \
         break;                                                                                              \
     }
     // Eight wavefronts (two per 16 queries, half a key tile each) shorten the longest workgroup's chain of
@@ -364,6 +389,7 @@ int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const vo
         default: return -1;
     }
 #undef PF_CASE
+#undef PF_LAUNCH
     MLLM_LAUNCH_CHECK();
     return 0;
 }

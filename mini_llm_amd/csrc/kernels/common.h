@@ -236,6 +236,16 @@ __device__ __forceinline__ void epilogue(int mode, float acc, float bias, void* 
     }
 }
 
+#include "score_shape.h"
+
+// A score (already times its scale, natural units) of query head with bias numbers r1, r2 at distance `dist`.
+__device__ __forceinline__ float mllm_shaped_score(float s, const MllmScoreShape& sh, float r1, float r2, int dist) {
+    if (sh.softcap > 0.f) s = sh.softcap * tanhf(s / sh.softcap);
+    if (sh.r1 != nullptr) s -= r1 * log1pf(r2 * static_cast<float>(dist));
+    return s;
+}
+#define MLLM_LOG2E 1.44269504088896340736f
+
 #define MLLM_LAUNCH_CHECK()                                   \
     do {                                                      \
         hipError_t e_ = hipGetLastError();                    \

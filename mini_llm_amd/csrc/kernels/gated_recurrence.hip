@@ -72,9 +72,9 @@ hgrn2_scan_kernel(const float* __restrict__ proj, int ld, int q_col, int f_col, 
     float s[GR_ROWS];
 #pragma unroll
     for (int i = 0; i < GR_ROWS; ++i) {
-        s[i] = 0.f;
-        if (MODE == 0 && i < rows && col_ok) s[i] = S[static_cast<size_t>(i) * dv];
-        if (MODE == 2 && i < rows && col_ok) s[i] = WS[static_cast<size_t>(i) * dv];
+        // (the start: the slot's state, zero, or what the pass over the chunks left for this chunk)
+        const float* from = MODE == 2 ? WS : S;
+        s[i] = (MODE != 1 && i < rows && col_ok) ? from[static_cast<size_t>(i) * dv] : 0.f;
     }
     // the channel this lane prepares: lanes 0..31 the gate of channel lane, lanes 32..63 the query of channel lane - 32
     const int ch = lane % GR_ROWS;

@@ -195,9 +195,30 @@ scored_attention_rows(const T* __restrict__ q, int ldq, const T* __restrict__ k_
     }
 }
 
+// x[t, c] *= sigmoid(gate[t, c])
+template <typename T>
+__global__ void gate_mul_kernel(T* __restrict__ x, int ldx, const float* __restrict__ gate, int ldg, int N, long long total) {
+    const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const long long t = i / N;
+    const int c = static_cast<int>(i % N);
+    x[t * ldx + c] = from_float<T>(to_float(x[t * ldx + c]) * sigmoid_of(gate[t * ldg + c]));
+}
+
 }  // namespace
 
 extern "C" {
+
+int mllm_gate_mul(void* x, int ldx, const float* gate, int ldg, int T, int N, int dtype, hipStream_t stream) {
+    if (T <= 0 || N <= 0) return 0;
+    const long long total = static_cast<long long>(T) * N;
+    const int blocks = static_cast<int>((total + 255) / 256);
+    if (dtype == MLLM_F32) gate_mul_kernel<float><<<blocks, 256, 0, stream>>>(static_cast<float*>(x), ldx, gate, ldg, N, total);
+    else gate_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>(static_cast<bf16_t*>(x), ldx, gate, ldg, N, total);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
 
 // -1: sizes the kernel refuses (an odd rot_dims, rot_dims > d, values from keys with dv != d, more LDS than a
 // workgroup has).

@@ -46,7 +46,11 @@ class AttentionArgsC(ctypes.Structure):
                 ("n_seqs", _i), ("max_blocks", _i), ("token_seq", _vp), ("positions", _vp), ("scale", _f),
                 ("window", _i), ("out", Tensor2), ("cu_q", _vp), ("ctx_len", _vp), ("max_q_len", _i),
                 ("max_ctx_len", _i), ("append", _i), ("k_col", _i), ("v_col", _i), ("slots", _vp),
-                ("n_single", _i), ("may_split", _i)]
+                ("n_single", _i), ("may_split", _i), ("shape", _vp), ("gate", _vp), ("gate_stride", _i)]
+
+
+class ScoreShapeC(ctypes.Structure):
+    _fields_ = [("softcap", _f), ("chunk", _i), ("r1", _vp), ("r2", _vp)]
 
 
 _lib = None
@@ -171,6 +175,12 @@ def reset_seen() -> None:
 def set_latent_tiles(on: bool) -> None:
     """Whether latent attention's prompt portions may run on the matrix cores (default: on)."""
     _ok(engine_library().mllm_set_tuning(b"latent_tiles", 1 if on else 0, 0))
+
+
+def set_scored_shared_kernels(on: bool) -> None:
+    """Whether attention with shaped scores may run on the kernels that plain attention runs on (default: on);
+    off: every row goes through the one-wavefront-per-row kernel that takes any sizes."""
+    _ok(engine_library().mllm_set_tuning(b"scored_shared_kernels", 1 if on else 0, 0))
 
 
 # Tuning hooks: tests and tuning scripts set these module attributes; they reach the native side at the
@@ -384,7 +394,8 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
                     block_tables: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor,
                     scale: float, window: int, out: torch.Tensor, *, cu_q: Optional[torch.Tensor] = None,
                     ctx_len: Optional[torch.Tensor] = None, max_q_len: int = 0, max_ctx_len: int = 0,
-                    append: Optional[tuple] = None, n_single: int = 0, may_split: bool = False):
+                    append: Optional[tuple] = None, n_single: int = 0, may_split: bool = False,
+                    shape: Optional[dict] = None, gate: Optional[torch.Tensor] = None):
     """Causal attention of the step's queries over the pages.
 
     q: [T, >= q_col + n_heads*head_dim] (queries of token t start at column q_col);
@@ -403,6 +414,11 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
     ``may_split``: the caller hands the result to ``linear`` next and accepts an ``AttentionSplits``
     in place of ``out`` (returned when a few single tokens' keys were split over several workgroups
     each; ``out`` is then left unwritten).
+
+    ``shape``: scores shaped before the softmax, ``{"softcap": c, "chunk": n, "r1": tensor, "r2": tensor}`` (any
+    subset): ``s <- c tanh(s / c)``, then ``s <- s - r1[h] ln(1 + r2[h] (i - j))`` (fp32 [n_heads] each), and with
+    ``chunk`` a query sees only the keys of its own block of n positions. ``gate`` (fp32 [T, n_heads*head_dim],
+    only with ``shape``): the result is multiplied by its sigmoid. Neither goes with ``append`` or ``may_split``.
     """
     _gpu(q, k_pages, v_pages, block_tables, token_seq, positions, out, cu_q, ctx_len)
     T = q.shape[0]
@@ -430,6 +446,25 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
         _i32(slots, "slots", T)
         a.append, a.k_col, a.v_col, a.slots = 1, int(k_col), int(v_col), slots.data_ptr()
     a.n_single, a.may_split = int(n_single), 1 if may_split else 0
+    sh = None
+    if shape is not None:
+        sh = ScoreShapeC()
+        sh.softcap, sh.chunk = float(shape.get("softcap") or 0.0), int(shape.get("chunk") or 0)
+        r1, r2 = shape.get("r1"), shape.get("r2")
+        if (r1 is None) != (r2 is None):
+            raise KernelError("the distance bias needs r1 and r2")
+        if r1 is not None:
+            _gpu(r1, r2)
+            for t_, n_ in ((r1, "r1"), (r2, "r2")):
+                if t_.dtype != torch.float32 or t_.numel() != n_heads or not t_.is_contiguous():
+                    raise KernelError(f"{n_} must be contiguous float32 [n_heads]")
+            sh.r1, sh.r2 = r1.data_ptr(), r2.data_ptr()
+        a.shape = ctypes.addressof(sh)
+    if gate is not None:
+        _gpu(gate)
+        if gate.dtype != torch.float32 or gate.dim() != 2 or gate.shape[0] != T or gate.shape[1] < n_heads * head_dim or gate.stride(1) != 1:
+            raise KernelError("gate must be float32 [T, >= n_heads*head_dim]")
+        a.gate, a.gate_stride = gate.data_ptr(), gate.stride(0)
     push_tuning()
     splits, unmerged = AttentionSplitsC(), _i(0)
     _ok(engine_library().mllm_op_paged_attention(ctypes.byref(a), ctypes.byref(splits), ctypes.byref(unmerged), _stream()))

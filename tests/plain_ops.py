@@ -90,7 +90,7 @@ def kv_append(src, k_col, v_col, kv_dim, k_pages, v_pages, slots):
 
 
 def paged_attention(q, q_col, n_heads, n_kv_heads, head_dim, k_pages, v_pages, page_size, block_tables,
-                    token_seq, positions, scale, window, out, append=None, **_):
+                    token_seq, positions, scale, window, out, append=None, shape=None, gate=None, **_):
     # (the hints n_single and may_split change nothing here: the result is always merged into `out`)
     T = q.shape[0]
     if append is not None:
@@ -99,6 +99,8 @@ def paged_attention(q, q_col, n_heads, n_kv_heads, head_dim, k_pages, v_pages, p
     for t in range(T):
         b, p = int(token_seq[t]), int(positions[t])
         lo = max(0, p - window + 1) if window else 0
+        if shape and shape.get("chunk"):
+            lo = p - p % shape["chunk"]           # only the keys of the query's own block of positions
         js = torch.arange(lo, p + 1)
         rows = block_tables[b].long()[js // page_size] * page_size + js % page_size
         for h in range(n_heads):
@@ -107,8 +109,15 @@ def paged_attention(q, q_col, n_heads, n_kv_heads, head_dim, k_pages, v_pages, p
             k = k_pages[rows, hk * head_dim:(hk + 1) * head_dim].to(PRECISE)
             v = v_pages[rows, hk * head_dim:(hk + 1) * head_dim].to(PRECISE)
             s = (k @ qv) * scale
+            if shape and shape.get("softcap"):
+                s = shape["softcap"] * torch.tanh(s / shape["softcap"])
+            if shape and shape.get("r1") is not None:
+                s = s - shape["r1"][h].to(PRECISE) * torch.log1p(shape["r2"][h].to(PRECISE) * (p - js).to(PRECISE))
             w = torch.softmax(s, dim=0)
-            out[t, h * head_dim:(h + 1) * head_dim] = (w @ v).to(out.dtype)
+            o = w @ v
+            if gate is not None:
+                o = o * torch.sigmoid(gate[t, h * head_dim:(h + 1) * head_dim].to(PRECISE))
+            out[t, h * head_dim:(h + 1) * head_dim] = o.to(out.dtype)
     return out
 
 

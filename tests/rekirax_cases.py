@@ -70,8 +70,22 @@ ODD = model([
     parallel(heads=2, kv_heads=2, dim=6, vdim=5, chunk=3, dims=0, r_heads=2, r_dim=5, r_vdim=9),
 ], vocab=101, width=44, taps=6, loop=(0, 1, 2))
 
+# head sizes and page sizes that the attention kernels shared with the other models take: 64 and 128 (the bfloat16
+# matrix-core kernel of prompt portions, the split-key kernel of single tokens), 48 (the 32-bit matrix-core tiles only);
+# windows and chunks shorter and longer than a tile of 64 or 128 keys, chunks that end inside a tile of queries
+SHARED_KERNELS = model([
+    parallel(heads=4, kv_heads=2, dim=64, vdim=64, chunk=100, dims=32, r_heads=2, r_dim=16, r_vdim=16, mlp=dense(64)),
+    attention(heads=2, kv_heads=1, dim=128, window=150, softcap=8.0),
+    parallel(heads=2, kv_heads=2, dim=128, vdim=128, chunk=37, dims=64, r_heads=1, r_dim=8, r_vdim=8),
+    attention(heads=3, kv_heads=3, dim=48, window=70, softcap=None),
+    attention(heads=4, kv_heads=1, dim=64, window=20, scale=0.5, softcap=4.0, mlp=dense(64)),
+], vocab=211, width=64, loop=(2, 4, 2))
+
 # rms(difference, mean taken off) / rms(logits, mean taken off) of a row may be at most this
-TOL = {"float32": 5e-6, "bfloat16": 6e-2}
+# (32-bit: the kernels shared with plain attention work in base 2, one more rounding of every score than the plain
+# model has; rows early in a sequence, where a head's recurrent output is still small in front of its unit norm,
+# show it most: 1e-5 was seen, 5e-6 through the row kernel)
+TOL = {"float32": 2e-5, "bfloat16": 6e-2}
 TOL_PEAKED = 1e-4
 
 _plain: Dict[tuple, np.ndarray] = {}

@@ -435,7 +435,7 @@ def test_kv_append_reference_vector(ops, dtype):
     assert (kp.cpu()[untouched] == -1).all() and (vp.cpu()[untouched] == -1).all()
 
 
-def _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, gen, boost=None, n_single=0):
+def _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, gen, boost=None, n_single=0, q_col=8, shape=None, gated=False):
     """seqs: list of (start, q_len). Builds pages in scrambled order, garbage elsewhere."""
     B = len(seqs)
     ctx = [s + n for s, n in seqs]
@@ -459,7 +459,7 @@ def _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, gen, boost=None,
         if boost is not None and ctx[b] > boost[0]:
             # one far key stands out: its score dominates for the last query
             far = boost[0]
-            k[far] = k[far] * 0 + (q[len(token_seq) + n - 1, 8:8 + H * dh].float().view(H, dh)[::H // Hkv]
+            k[far] = k[far] * 0 + (q[len(token_seq) + n - 1, q_col:q_col + H * dh].float().view(H, dh)[::H // Hkv]
                                    .reshape(-1) * boost[1]).to(dtype)
         js = torch.arange(ctx[b])
         rows = tables[b].long()[js // page] * page + js % page
@@ -472,13 +472,19 @@ def _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, gen, boost=None,
     scale = dh ** -0.5
     out = torch.zeros(T, H * dh, dtype=dtype, device=DEV)
     cu = torch.tensor([0] + list(torch.tensor([n for _, n in seqs]).cumsum(0)), dtype=torch.int32)
-    ops.paged_attention(q.to(DEV), 8, H, Hkv, dh, kp.to(DEV), vp.to(DEV), page, tables.to(DEV),
+    gate = torch.randn(T, H * dh + 4, generator=gen) * 2 if gated else None
+    on_dev = None
+    if shape is not None:
+        on_dev = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in shape.items()}
+    ops.paged_attention(q.to(DEV), q_col, H, Hkv, dh, kp.to(DEV), vp.to(DEV), page, tables.to(DEV),
                         token_seq.to(DEV), positions.to(DEV), scale, window, out,
                         cu_q=cu.to(DEV), ctx_len=torch.tensor(ctx, dtype=torch.int32).to(DEV),
-                        max_q_len=max(n for _, n in seqs), max_ctx_len=max(ctx), n_single=n_single)
+                        max_q_len=max(n for _, n in seqs), max_ctx_len=max(ctx), n_single=n_single,
+                        shape=on_dev, gate=gate.to(DEV) if gated else None)
     ref = torch.zeros(T, H * dh, dtype=torch.float64)
-    plain_ops.paged_attention(q, 8, H, Hkv, dh, kp, vp, page, tables, token_seq, positions, scale, window, ref)
-    if sum(c * n for c, (_, n) in zip(ctx, seqs)) * H * dh <= 2e8:
+    plain_ops.paged_attention(q, q_col, H, Hkv, dh, kp, vp, page, tables, token_seq, positions, scale, window, ref,
+                              shape=shape, gate=gate)
+    if shape is None and sum(c * n for c, (_, n) in zip(ctx, seqs)) * H * dh <= 2e8:
         # the second oracle, the plain C++ twin, says the same
         twin = ref_ops.paged_attention(q, 8, H, Hkv, dh, kp, vp, page, tables, token_seq, positions, scale, window)
         assert (twin.double() - ref).abs().max() <= 2e-6
@@ -519,6 +525,31 @@ def test_paged_attention_decode_only(ops, dtype, H, Hkv, dh, page, window, shape
         assert (out - ref).abs().max() <= _tol(dtype, 2)
     finally:
         ops.DECODE_SHAPE_OVERRIDE = None
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,dh,page", [(4, 2, 64, 16), (6, 2, 128, 16), (3, 3, 32, 8), (5, 5, 48, 16), (2, 1, 40, 4)])
+@pytest.mark.parametrize("kind", ["window_bias", "chunk_gate"])
+def test_paged_attention_with_shaped_scores(ops, dtype, H, Hkv, dh, page, kind):
+    """Scores capped and biased by the distance under a sliding window, or a chunked mask with a gate on the result,
+    on every kernel of the dispatch: prompt portions (matrix-core tiles in bfloat16 and in 32-bit; the row kernel for
+    a head of 40), single tokens (split keys), and a mixed step whose single tokens stand in front. One far key is
+    boosted so that a lost key, a chunk's or a window's edge one off shows."""
+    g = torch.Generator().manual_seed(H * 7 + dh + len(kind))
+    if kind == "window_bias":
+        window = 150
+        shape = {"softcap": 6.0, "r1": torch.rand(H, generator=g) + 0.2, "r2": torch.rand(H, generator=g) + 0.1}
+    else:
+        window = 0
+        shape = {"chunk": 70}
+    gated = kind == "chunk_gate"
+    cases = [([(0, 37), (130, 70), (64, 2), (5, 300)], 0), ([(1023, 1), (0, 1), (63, 1), (149, 1), (150, 1), (69, 1), (70, 1), (500, 1)], 8),
+             ([(300, 1), (12, 1), (0, 100), (200, 64), (139, 1)], 2)]
+    for seqs, n_single in cases:
+        out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, g, boost=(max(0, seqs[0][0] + seqs[0][1] - 3), 0.5),
+                                   n_single=n_single, q_col=0, shape=shape, gated=gated)
+        assert torch.isfinite(out).all()
+        assert (out - ref).abs().max() <= _tol(dtype, 2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -70,6 +70,47 @@ def test_schedule_families_match_plain(dirs, name, family, dtype):
     assert runner.check() == "" and info["free_pages"] == n_pages and info["n_requests"] == 0
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page", [8, 16, 64])
+@pytest.mark.parametrize("family", ["whole", "decode", "chunks", "mixed"])
+def test_on_the_kernels_shared_with_plain_attention(dirs, family, page, dtype):
+    """Head sizes 64, 128 and 48 at pages of 8 to 64 tokens: prompt portions on the matrix-core tiles, single tokens on
+    the split-key kernel, with shaped scores, chunks and gates handed on; prompts of up to 300 tokens (several key
+    tiles, windows and chunks that end inside a tile), portions, and mixed batches whose single tokens ride along."""
+    from mini_llm_amd.kernels import ops
+    cfg, d = rc.SHARED_KERNELS, dirs("SHARED_KERNELS")
+    reqs = rc.requests(cfg["vocab"], [1, 2, 17, 63, 64, 65, 130, 300], seed=71)
+    steps = _families(reqs, seed=6)[family]
+    ops.reset_seen()
+    runner = _runner(d, dtype, n_pages=-(-ru.peak_tokens(steps) // page), page=page)
+    rc.check_against_plain(d, reqs, steps, ru.run_in_process(runner, steps), dtype, cfg["vocab"], f"shared kernels page {page} {family}")
+    if family == "whole":
+        assert ops.seen("prefill_tile_launches" if dtype == "bfloat16" else "tiled_f32_launches") > 0
+    assert runner.check() == "" and runner.info()["n_requests"] == 0
+
+
+def test_shared_kernels_against_the_row_kernel(dirs):
+    """The same steps with the shared kernels switched off (every row through the one-wavefront-per-row kernel):
+    both round differently, no more."""
+    from mini_llm_amd.kernels import ops
+    cfg, d = rc.SHARED_KERNELS, dirs("SHARED_KERNELS")
+    reqs = rc.requests(cfg["vocab"], [5, 100, 257], seed=72)
+    steps, _ = ru.trace_mixed(reqs, seed=9, max_live=3, tail=20)
+    got = []
+    try:
+        for on in (True, False):
+            ops.set_scored_shared_kernels(on)
+            ops.reset_seen()
+            runner = _runner(d, "float32", n_pages=ru.peak_tokens(steps) // 16, page=16)
+            got.append(ru.collect(steps, ru.run_in_process(runner, steps), cfg["vocab"]))
+            assert (ops.seen("tiled_f32_launches") > 0) == on
+    finally:
+        ops.set_scored_shared_kernels(True)
+    worst = max(rc.row_error(got[0][r][p], got[1][r][p].astype(np.float64)) for r in reqs for p in range(len(reqs[r])))
+    print(f"shared kernels against the row kernel: {worst:.3e}")
+    assert worst <= 2e-5
+
+
 @pytest.mark.parametrize("page", [2, 4, 16])
 def test_window_chunk_and_page_borders_with_peaked_scores(dirs, page):
     """Scores scaled so that single keys dominate, windows of 5 and 16 and chunks of 6 over pages of 2, 4 and 16
