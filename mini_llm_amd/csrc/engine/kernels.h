@@ -56,7 +56,8 @@ int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_
                           const int* positions, int n_q, int n_heads, int n_kv_heads, int head_dim,
                           int page_size, float scale, int window, int nsplit, int waves, void* out,
                           int out_stride, float* ws, int* counters, int k_col, int v_col, const int* slots,
-                          int partial_out, int dtype, hipStream_t stream, const MllmScoreShape* shape = nullptr);
+                          int partial_out, int dtype, hipStream_t stream, const MllmScoreShape* shape = nullptr,
+                          const float* gate = nullptr, int ldg = 0);
 int mllm_merge_attention_splits(const float* ws, int n_q, int n_heads, int head_dim, int nsplit, void* out,
                                 int out_stride, int dtype, hipStream_t stream);
 int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
@@ -70,6 +71,8 @@ int mllm_rmsnorm(const float* x, int ldx, const int* rows, const float* w, const
                  int n, int D, int groups, float eps, int out_dtype, int parts, size_t part_stride, hipStream_t stream);
 int mllm_rmsnorm_add(float* y, const float* w, const float* scale, float mult, float eps, float* x, int n, int D,
                      int clear, hipStream_t stream);
+int mllm_rmsnorm_add_many(const float* y, size_t y_stride, const float* w, size_t w_stride, int n_in, float mult, float eps,
+                          float* x, int n, int D, hipStream_t stream);
 int mllm_glu_clamped(const void* gate, int ldg, const void* up, int ldu, void* out, int ldo, int T, int F, float limit,
                      float alpha, int dtype, hipStream_t stream);
 int mllm_fill_zero(void* p, size_t bytes, hipStream_t stream);
@@ -81,6 +84,9 @@ int mllm_conv_silu(const float* proj, int ld, int col0, int C, const float* w, c
 int mllm_conv_residual(const float* in, int ld, int C, const float* w, int taps, const int* token_seq, const int* cu_q,
                        const int* state_slots, float* state, size_t slot_floats, void* out, int ldo, int out_dtype, int T,
                        int B, int write, hipStream_t stream);
+int mllm_rmsnorm_conv_single(const float* x, int ldx, const float* wn, float eps, int C, const float* wc, int taps,
+                             const int* state_slots, float* state, size_t slot_floats, void* out, int ldo, int out_dtype, int T,
+                             int write, hipStream_t stream);
 int mllm_ssm_scan(const float* xbc, int ldx, const float* raw_dt, int ldd, const float* dt_bias, const float* A_log,
                   const float* Dskip, const int* cu_q, const int* state_slots, float* state, size_t slot_floats,
                   size_t scan_offset, float* y, int ldy, size_t part_stride, int T, int B, int max_q_len, int H, int P, int N,

@@ -486,13 +486,15 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
                                     a.block_tables, a.max_blocks, seq_of_token, a.positions, T, a.n_heads, a.n_kv_heads,
                                     a.head_dim, a.page_size, a.scale, a.window, nsplit, waves, a.out.data,
                                     static_cast<int>(a.out.stride), ws, counters, a.k_col, a.v_col, slots,
-                                    unmerged || merge_kernel ? 1 : 0, a.q.dtype, stream, a.shape), "decode_attention");
+                                    unmerged || merge_kernel ? 1 : 0, a.q.dtype, stream, a.shape, merge_kernel ? nullptr : a.gate, a.gate_stride),
+              "decode_attention");
         tuning().seen.max_decode_splits = std::max(tuning().seen.max_decode_splits, nsplit);
         if (merge_kernel) tuning().seen.merge_kernel_launches += 1;
         if (merge_kernel)
             check(mllm_merge_attention_splits(ws, T, a.n_heads, a.head_dim, nsplit, a.out.data, static_cast<int>(a.out.stride),
                                               a.q.dtype, stream), "merge_splits");
-        if (a.gate != nullptr)
+        // (a result that the merge kernel finishes takes its gate in a kernel of its own)
+        if (a.gate != nullptr && merge_kernel)
             check(mllm_gate_mul(a.out.data, static_cast<int>(a.out.stride), a.gate, a.gate_stride, T, q_dim, a.q.dtype, stream), "gate_mul");
         if (unmerged) {
             splits->ws = ws;

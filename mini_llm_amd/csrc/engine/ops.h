@@ -248,6 +248,14 @@ void latent_expand(const Tensor2& o_lat, const Tensor2& w_uv, const Tensor2& out
 // out = in + conv(in): a causal convolution per channel over `taps` inputs (taps [channels, taps], the last tap
 // the token's own), added onto its input; in fp32 [T, C], out in its own dtype. Carried inputs as for conv_silu.
 void conv_residual(const Tensor2& in, const Tensor2& weight, const StateArgs& st, const Tensor2& out, hipStream_t stream);
+// The same behind an RMS norm, in one kernel, for a step in which every sequence brings one token (x.rows == st.n_seqs):
+// out = h + conv(h) with h = x / sqrt(mean(x^2) + eps) * norm_weight.
+// False (and nothing done): sizes the kernel is not made for (more than 8 taps, rows wider than 2,048).
+bool rmsnorm_conv_single(const Tensor2& x, const float* norm_weight, float eps, const Tensor2& weight, const StateArgs& st,
+                         const Tensor2& out, hipStream_t stream);
+// x += mult * sum_k rmsnorm(y_k) * w_k: n inputs of x's shape one behind the other in `ys` ([n * rows, size] fp32), their
+// weights one behind the other in `weights` ([n * size]); 2 to 4 inputs, rows of up to 2,048 columns.
+void rmsnorm_add_many(const Tensor2& ys, const float* weights, int n, float mult, float eps, const Tensor2& x, hipStream_t stream);
 // Sizes and constants of an attention whose scores are shaped before the softmax (kernels/scored_attention.hip).
 struct ScoredShape {
     int n_heads = 0, n_kv_heads = 0, dim = 0, value_dim = 0;

@@ -53,6 +53,33 @@ void conv_residual(const Tensor2& in, const Tensor2& weight, const StateArgs& st
                              st.write ? 1 : 0, stream), "conv_residual");
 }
 
+bool rmsnorm_conv_single(const Tensor2& x, const float* norm_weight, float eps, const Tensor2& weight, const StateArgs& st,
+                         const Tensor2& out, hipStream_t stream) {
+    need_f32(x, "rmsnorm_conv_single: the input");
+    need_f32(weight, "rmsnorm_conv_single: the taps");
+    need_act(out, "rmsnorm_conv_single: out");
+    const int C = i32(weight.rows), taps = i32(weight.cols);
+    if (!weight.contiguous() || taps < 1 || taps > 16 || norm_weight == nullptr) fail("rmsnorm_conv_single: taps [channels, 1 to 16] contiguous and the norm's weight are needed");
+    if (x.cols != C || out.cols != C || out.rows != x.rows) fail("rmsnorm_conv_single: input and out must be [T, %d]", C);
+    if (x.rows != st.n_seqs || st.state_slots == nullptr) fail("rmsnorm_conv_single: every sequence of the step must bring one token");
+    if (taps > 1 && (st.state == nullptr || st.slot_floats < static_cast<size_t>(taps - 1) * C))
+        fail("rmsnorm_conv_single: a state slot holds %zu floats, %zu are needed", st.slot_floats, static_cast<size_t>(taps - 1) * C);
+    const int rc = mllm_rmsnorm_conv_single(static_cast<const float*>(x.data), i32(x.stride), norm_weight, eps, C, static_cast<const float*>(weight.data), taps,
+                                            st.state_slots, st.state, st.slot_floats, out.data, i32(out.stride), out.dtype, i32(x.rows), st.write ? 1 : 0, stream);
+    if (rc == -2) return false;
+    check(rc, "rmsnorm_conv_single");
+    return true;
+}
+
+void rmsnorm_add_many(const Tensor2& ys, const float* weights, int n, float mult, float eps, const Tensor2& x, hipStream_t stream) {
+    need_f32(ys, "rmsnorm_add_many: the inputs");
+    need_f32(x, "rmsnorm_add_many: x");
+    if (n < 2 || n > 4 || weights == nullptr || x.cols > 2048) fail("rmsnorm_add_many: two to four inputs with their weights, rows of up to 2,048 columns");
+    if (!ys.contiguous() || !x.contiguous() || ys.rows != x.rows * n || ys.cols != x.cols) fail("rmsnorm_add_many: the inputs must be [%d * rows, size] beside x [rows, size]", n);
+    check(mllm_rmsnorm_add_many(static_cast<const float*>(ys.data), static_cast<size_t>(x.rows) * x.cols, weights, static_cast<size_t>(x.cols), n, mult, eps,
+                                static_cast<float*>(x.data), i32(x.rows), i32(x.cols), stream), "rmsnorm_add_many");
+}
+
 void qk_prepare(const Tensor2& proj, int q_col, int k_col, int v_col, const ScoredShape& sh, const int* positions,
                 const int* slots, const Tensor2& q, const Tensor2& k_pages, const Tensor2& v_pages, hipStream_t stream) {
     check_shape(sh, "qk_prepare");

@@ -332,14 +332,18 @@ public:
         if (conv_.data != nullptr) {
             if (conv_bytes_ > 0 && (!cache.has_state() || cache.state_bytes < conv_bytes_)) fail("a block with an input convolution needs %zu bytes of state per request", conv_bytes_);
             if (x.cols != conv_.rows) fail("the input convolution has %lld channels, the stream %lld", (long long)conv_.rows, (long long)x.cols);
-            Tensor2 hn = arena.tensor(F32, x.rows, x.cols);      // the convolution reads the normed rows in fp32
-            norm1_->forward_into(x, nullptr, hn, s);
             Tensor2 hc = arena.tensor(dtype_, x.rows, x.cols);
             StateArgs st;
             st.token_seq = step.token_seq; st.cu_q = step.cu_q; st.state_slots = step.state_slots; st.n_seqs = step.n_seqs;
             st.max_q_len = step.max_q_len; st.state = static_cast<float*>(cache.state); st.slot_floats = cache.slot_bytes / 4;
             st.n_slots = cache.n_slots; st.write = write;
-            conv_residual(hn, conv_, st, hc, s);
+            // every sequence brings one token: norm and convolution in one kernel, if the norm has it
+            const bool single = step.max_q_len == 1 && step.n_tokens == step.n_seqs;
+            if (!(single && norm1_->conv_single(x, conv_, st, hc, s))) {
+                Tensor2 hn = arena.tensor(F32, x.rows, x.cols);      // the convolution reads the normed rows in fp32
+                norm1_->forward_into(x, nullptr, hn, s);
+                conv_residual(hn, conv_, st, hc, s);
+            }
             StageTimes::get().mark("input_conv", s);
             CacheView rest = cache;                     // what lies behind the carried rows is the mixer's
             if (conv_bytes_ > 0) {

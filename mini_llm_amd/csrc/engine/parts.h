@@ -205,6 +205,13 @@ public:
     // out[i,:] = norm(x[rows ? rows[i] : i, :]) into a tensor of the caller's (any activation dtype; out may be x
     // itself when rows is null and both are fp32). A norm without it refuses.
     virtual void forward_into(const Tensor2& x, const int* rows, const Tensor2& out, hipStream_t s) const;
+    // For a step in which every sequence brings one token: out = h + conv(h) with h = norm(x), the convolution's
+    // earlier inputs carried in the slots (StateArgs), in one kernel. False: this kind of norm has no such kernel,
+    // and nothing was done.
+    virtual bool conv_single(const Tensor2& x, const Tensor2& taps, const StateArgs& st, const Tensor2& out, hipStream_t s) const {
+        (void)x; (void)taps; (void)st; (void)out; (void)s;
+        return false;
+    }
     // out = epilogue(lin(norm(x[rows]))); a norm with a fused kernel overrides this
     // (kv: a key/value scatter of the linear map, passed through to it)
     virtual void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,

@@ -32,6 +32,10 @@ public:
         if (x.cols != size_) fail("rmsnorm: rows of %lld, the norm is %d wide", (long long)x.cols, size_);
         rmsnorm(x, weight_, eps_, 1, nullptr, out, rows, s);
     }
+    bool conv_single(const Tensor2& x, const Tensor2& taps, const StateArgs& st, const Tensor2& out, hipStream_t s) const override {
+        if (x.cols != size_) fail("rmsnorm: rows of %lld, the norm is %d wide", (long long)x.cols, size_);
+        return rmsnorm_conv_single(x, weight_, eps_, taps, st, out, s);
+    }
     void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,
                 const KvScatter* kv, Arena& arena, hipStream_t s) const override {
         if (kv != nullptr) { Norm::linear(x, lin, out, epilogue, rows, kv, arena, s); return; }

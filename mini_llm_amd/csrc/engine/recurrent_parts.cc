@@ -89,7 +89,8 @@ private:
 // Mixers side by side on the same input: x += (1 / n) sum_k rmsnorm(mixer_k(h)) * weight_k, every mixer's output
 // RMS-normed over the stream's width with a weight of its own before the mean is taken. Each mixer adds into a
 // cleared fp32 buffer of the stream's shape. At most one of them may keep pages; their states lie one behind the
-// other in the layer's state slot. Parameters: size, eps; mixers; tensors norm0, norm1, ...
+// other in the layer's state slot. Parameters: size, eps; mixers; tensors norm0, norm1, ... and optionally
+// norms (the same weights one behind the other: the norms and the mean then run in one kernel).
 class ParallelMixers final : public Mixer {
 public:
     explicit ParallelMixers(const Params& p) : mixers_(p.mixers) {
@@ -103,6 +104,12 @@ public:
             if (mixers_[k]->cache_need().kind & 1) with_pages += 1;
         }
         if (with_pages > 1) fail("parallel mixers: only one of the mixers may keep pages");
+        // (the weights one behind the other in one tensor: all norms and the mean in one kernel)
+        if (const Tensor2* j = p.weights_or_null("norms")) {
+            if (j->dtype != F32 || !j->contiguous() || j->rows * j->cols != static_cast<int64_t>(size_) * static_cast<int64_t>(mixers_.size()))
+                fail("parallel mixers: 'norms' must be contiguous float32 [%zu * %d]", mixers_.size(), size_);
+            joined_norms_ = static_cast<const float*>(j->data);
+        }
     }
     void forward(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write, Arena& arena,
                  hipStream_t s) const override {
@@ -130,7 +137,8 @@ public:
             mixers_[k]->forward(h, step, mine, all.row_range(x.rows * k, x.rows), write, arena, s);
             arena.release(mark);
         }
-        for (int k = 0; k < n; ++k) rmsnorm_add(all.row_range(x.rows * k, x.rows), norms_[k], nullptr, 1.0f / n, eps_, x, false, s);
+        if (joined_norms_ != nullptr && n <= 4 && x.cols <= 2048) rmsnorm_add_many(all, joined_norms_, n, 1.0f / n, eps_, x, s);
+        else for (int k = 0; k < n; ++k) rmsnorm_add(all.row_range(x.rows * k, x.rows), norms_[k], nullptr, 1.0f / n, eps_, x, false, s);
         StageTimes::get().mark("mix", s);
     }
     size_t workspace_bytes(int tokens) const override {
@@ -157,6 +165,7 @@ public:
 private:
     std::vector<std::shared_ptr<const Mixer>> mixers_;
     std::vector<const float*> norms_;
+    const float* joined_norms_ = nullptr;
     int size_ = 0;
     float eps_ = 1e-6f;
 };

@@ -282,6 +282,7 @@ void rekirax_assemble(const Json& config, const std::map<std::string, Tensor2>& 
             pp.mixers.push_back(std::shared_ptr<const Mixer>(attention_mixer(l.att, M + "left.", true, c.eps, dtype, t, out.store).release()));
             pp.mixers.push_back(std::shared_ptr<const Mixer>(build_mixer("hgrn2", rp).release()));
             pp.tensor["norm0"] = t.at(M + "left.out"); pp.tensor["norm1"] = t.at(R + "out");
+            pp.tensor["norms"] = out.store.join_rows({t.at(M + "left.out"), t.at(R + "out")});
             mixer = build_mixer("parallel", pp);
         }
         std::unique_ptr<FeedForward> ff;

@@ -237,7 +237,7 @@ paged_attention_tiled(const T* __restrict__ q, int q_stride, int q_col, const T*
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int j = k0 + 16 * g + 4 * G + i;
-                if (SHAPED) s[g][i] = mllm_shaped_score(s[g][i], shape, r1, r2, max(p - j, 0)) * MLLM_LOG2E;
+                if (SHAPED) s[g][i] = mllm_shaped_score<sizeof(T) == 2>(s[g][i], shape, r1, r2, max(p - j, 0)) * MLLM_LOG2E;
                 s[g][i] = (j <= p && j >= my_lo) ? s[g][i] : -INFINITY;
                 mx = fmaxf(mx, s[g][i]);
             }

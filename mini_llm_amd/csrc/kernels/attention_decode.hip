@@ -75,7 +75,8 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
                         float scale_log2e, T* __restrict__ out, int out_stride,
                         float* __restrict__ ws_o, float* __restrict__ ws_ml, int* __restrict__ counters,
                         T* __restrict__ k_pages_w, T* __restrict__ v_pages_w, int k_col, int v_col,
-                        const int* __restrict__ slots, int partial_out, MllmScoreShape shape) {
+                        const int* __restrict__ slots, int partial_out, MllmScoreShape shape,
+                        const float* __restrict__ gate, int ldg) {
     constexpr int EPL = Vec16<T>::N;        // elements per lane
     constexpr int DH = LPK * EPL;           // head size
     constexpr int KPW = MLLM_WAVE / LPK;    // keys per wavefront and load instruction
@@ -178,7 +179,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
             for (int e = 0; e < EPL; ++e) d = fmaf(qf[e], kf[e], d);
             d = group_sum<LPK>(d);
             const bool valid = j0 + u * group_keys + g < ke_pages;
-            if (SHAPED) d = mllm_shaped_score(d, shape, r1, r2, valid ? p - (j0 + u * group_keys + g) : 0) * MLLM_LOG2E;
+            if (SHAPED) d = mllm_shaped_score<sizeof(T) == 2>(d, shape, r1, r2, valid ? p - (j0 + u * group_keys + g) : 0) * MLLM_LOG2E;
             dot[u] = valid ? d : NEG;
             mx = fmaxf(mx, dot[u]);
         }
@@ -207,7 +208,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
 #pragma unroll
         for (int e = 0; e < EPL; ++e) d = fmaf(qf[e], kf[e], d);
         d = group_sum<LPK>(d);
-        if (SHAPED) d = mllm_shaped_score(d, shape, r1, r2, 0) * MLLM_LOG2E;
+        if (SHAPED) d = mllm_shaped_score<sizeof(T) == 2>(d, shape, r1, r2, 0) * MLLM_LOG2E;
         const float mn = fmaxf(m, d);
         const float a = exp2_for<T>(m - mn), pj = exp2_for<T>(d - mn);
         l = l * a + pj;
@@ -271,7 +272,11 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
         if (wave == 0 && g == 0) {
             const float inv = 1.0f / l;
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) op[e] = from_float<T>(o[e] * inv);
+            for (int e = 0; e < EPL; ++e) {
+                float r = o[e] * inv;
+                if (SHAPED && gate != nullptr) r *= 1.f / (1.f + __expf(-gate[static_cast<size_t>(t) * ldg + h * DH + c * EPL + e]));
+                op[e] = from_float<T>(r);
+            }
         }
         return;
     }
@@ -316,7 +321,11 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
     if (wave == 0 && g == 0) {
         const float inv = 1.0f / l;
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) op[e] = from_float<T>(o[e] * inv);
+        for (int e = 0; e < EPL; ++e) {
+            float r = o[e] * inv;
+            if (SHAPED && gate != nullptr) r *= 1.f / (1.f + __expf(-gate[static_cast<size_t>(t) * ldg + h * DH + c * EPL + e]));
+            op[e] = from_float<T>(r);
+        }
     }
     if (threadIdx.x == 0) counters[pair] = 0;     // ready for the next launch
 }
@@ -327,11 +336,12 @@ static int launch_decode(int lpk, dim3 grid, int waves, hipStream_t stream, cons
                          int max_blocks, const int* token_seq, const int* positions, int n_heads,
                          int n_kv_heads, int page_size, float scale_log2e, int window, int nsplit, T* out,
                          int out_stride, float* ws_o, float* ws_ml, int* counters, T* k_pages_w, T* v_pages_w,
-                         int k_col, int v_col, const int* slots, int partial_out, const MllmScoreShape* shape) {
+                         int k_col, int v_col, const int* slots, int partial_out, const MllmScoreShape* shape,
+                         const float* gate, int ldg) {
     const MllmScoreShape sh = shape ? *shape : MllmScoreShape{0.f, 0, nullptr, nullptr};
 #define DEC_ARGS token_seq, positions, block_tables, max_blocks, n_heads, n_kv_heads, page_size, window,  \
             nsplit, q, q_stride, q_col, k_pages, v_pages, kv_dim, scale_log2e, out, out_stride,        \
-            ws_o, ws_ml, counters, k_pages_w, v_pages_w, k_col, v_col, slots, partial_out, sh
+            ws_o, ws_ml, counters, k_pages_w, v_pages_w, k_col, v_col, slots, partial_out, sh, gate, ldg
 #define DEC_CASE(L)                                                                                    \
     case L:                                                                                            \
         if (shape) decode_attention_kernel<T, L, 8, true><<<grid, waves * MLLM_WAVE, 0, stream>>>(DEC_ARGS); \
@@ -409,7 +419,7 @@ int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_
                           const int* positions, int n_q, int n_heads, int n_kv_heads, int head_dim,
                           int page_size, float scale, int window, int nsplit, int waves, void* out,
                           int out_stride, float* ws, int* counters, int k_col, int v_col, const int* slots,
-                          int partial_out, int dtype, hipStream_t stream, const MllmScoreShape* shape) {
+                          int partial_out, int dtype, hipStream_t stream, const MllmScoreShape* shape, const float* gate, int ldg) {
     if (n_q <= 0) return 0;
     const int esz = dtype == MLLM_F32 ? 4 : 2;
     const int lpk = head_dim * esz / 16;
@@ -422,17 +432,19 @@ int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_
     // (shaped scores: the queries times the scale alone; the kernel goes to base 2 after the shaping)
     const float sl2 = shape ? scale : scale * 1.44269504088896340736f;
     if (shape && window > 0 && shape->chunk > 0) return -1;
+    // (a gate goes with shaped scores, and with a result that this kernel finishes itself)
+    if (gate != nullptr && (shape == nullptr || partial_out)) return -1;
     int rc;
     if (dtype == MLLM_F32)
         rc = launch_decode<float>(lpk, grid, waves, stream, (const float*)q, q_stride, q_col, (const float*)k_pages,
                                   (const float*)v_pages, kv_dim, block_tables, max_blocks, token_seq, positions,
                                   n_heads, n_kv_heads, page_size, sl2, window, nsplit, (float*)out, out_stride,
-                                  ws_o, ws_ml, counters, (float*)k_pages, (float*)v_pages, k_col, v_col, slots, partial_out, shape);
+                                  ws_o, ws_ml, counters, (float*)k_pages, (float*)v_pages, k_col, v_col, slots, partial_out, shape, gate, ldg);
     else
         rc = launch_decode<bf16_t>(lpk, grid, waves, stream, (const bf16_t*)q, q_stride, q_col, (const bf16_t*)k_pages,
                                    (const bf16_t*)v_pages, kv_dim, block_tables, max_blocks, token_seq, positions,
                                    n_heads, n_kv_heads, page_size, sl2, window, nsplit, (bf16_t*)out, out_stride,
-                                   ws_o, ws_ml, counters, (bf16_t*)k_pages, (bf16_t*)v_pages, k_col, v_col, slots, partial_out, shape);
+                                   ws_o, ws_ml, counters, (bf16_t*)k_pages, (bf16_t*)v_pages, k_col, v_col, slots, partial_out, shape, gate, ldg);
     if (rc != 0) return rc;
     MLLM_LAUNCH_CHECK();
     return 0;

@@ -191,7 +191,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
             for (int r = 0; r < 4; ++r) {
                 s[nt][r] = acc[r];                   // raw dot product; the scale is applied with the exponent
                 const int j = j_base + 16 * (nt0 + nt) + 4 * G + r;
-                if (SHAPED) s[nt][r] = mllm_shaped_score(acc[r] * scale, shape, r1, r2, max(p - j, 0)) * MLLM_LOG2E;
+                if (SHAPED) s[nt][r] = mllm_shaped_score<true>(acc[r] * scale, shape, r1, r2, max(p - j, 0)) * MLLM_LOG2E;
                 if (MASKED) {
                     const bool seen = q_ok && j <= p && (window <= 0 || j > p - window) && (chunk <= 0 || j >= p - p % chunk);
                     if (!seen) s[nt][r] = -INFINITY;

@@ -239,9 +239,18 @@ __device__ __forceinline__ void epilogue(int mode, float acc, float bias, void* 
 #include "score_shape.h"
 
 // A score (already times its scale, natural units) of query head with bias numbers r1, r2 at distance `dist`.
+// FAST (the bfloat16 kernels): tanh through one hardware exponential and a reciprocal, the logarithm by the hardware
+// instruction (at distance 0 its argument is exactly 1); otherwise the library's full-precision functions.
+template <bool FAST = false>
 __device__ __forceinline__ float mllm_shaped_score(float s, const MllmScoreShape& sh, float r1, float r2, int dist) {
-    if (sh.softcap > 0.f) s = sh.softcap * tanhf(s / sh.softcap);
-    if (sh.r1 != nullptr) s -= r1 * log1pf(r2 * static_cast<float>(dist));
+    if (sh.softcap > 0.f) {
+        const float u = s / sh.softcap;
+        s = sh.softcap * (FAST ? 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __expf(2.f * u)) : tanhf(u));
+    }
+    if (sh.r1 != nullptr) {
+        const float a = r2 * static_cast<float>(dist);
+        s -= r1 * (FAST ? __logf(1.f + a) : log1pf(a));
+    }
     return s;
 }
 #define MLLM_LOG2E 1.44269504088896340736f

@@ -82,12 +82,23 @@ hgrn2_scan_kernel(const float* __restrict__ proj, int ld, int q_col, int f_col, 
     const int c = h * d + i0 + (ch_ok ? ch : 0);
     const float lo = lower[c], fb = f_bias ? f_bias[c] : 0.f;
     float cum = 1.f;                            // (lanes 0..31) the product of the channel's gates over the chunk
+    // A token's inputs are asked for one token ahead (from a clamped, always valid row), so that the round trip to
+    // memory runs beside the arithmetic of the token before.
+    const int col = lane < GR_ROWS ? f_col + c : q_col + c;
+    const int vcol = v_col + h * dv + (col_ok ? e : 0);
+    float raw = 0.f, v_next = 0.f;
+    if (n > 0) {
+        raw = proj[static_cast<size_t>(first) * ld + col];
+        v_next = proj[static_cast<size_t>(first) * ld + vcol];
+    }
     for (int k = 0; k < n; ++k) {
-        const float* row = proj + static_cast<size_t>(first + k) * ld;
+        const float z = raw, v = col_ok ? v_next : 0.f;
+        const float* ahead = proj + static_cast<size_t>(first + min(k + 1, n - 1)) * ld;
+        raw = ahead[col];
+        v_next = ahead[vcol];
         float val;
-        if (lane < GR_ROWS) { val = lo + (1.f - lo) * gr_sigmoid(row[f_col + c] + fb); cum *= val; }
-        else { const float z = row[q_col + c]; val = z * gr_sigmoid(z); }
-        const float v = col_ok ? row[v_col + h * dv + e] : 0.f;
+        if (lane < GR_ROWS) { val = lo + (1.f - lo) * gr_sigmoid(z + fb); cum *= val; }
+        else val = z * gr_sigmoid(z);
         float* cur = fq[k & 1];
         cur[lane] = ch_ok ? val : 0.f;
         wave_lds_sync();

@@ -99,6 +99,56 @@ rmsnorm_add_kernel(float* __restrict__ y, const float* __restrict__ w, const flo
     }
 }
 
+// x[r, i] += mult * sum_k y_k[r, i] / sqrt(mean(y_k[r]^2) + eps) * w_k[i] for n inputs of x's shape that lie
+// y_stride floats apart (weights w_stride apart), added in the order of k; one wavefront per row.
+// N_IN inputs, NB blocks of 512 columns: every input row stays in registers between its statistics and the sum; loads
+// without conditions, from clamped places, masked where they are used.
+template <int WAVES, int N_IN, int NB>
+__global__ void __launch_bounds__(64 * WAVES)
+rmsnorm_add_many_kernel(const float* __restrict__ y, size_t y_stride, const float* __restrict__ w, size_t w_stride,
+                        float mult, float eps, float* __restrict__ x, int n, int D) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
+    const int r = blockIdx.x * WAVES + wave;
+    if (r >= n) return;
+    float v[N_IN][NB][8], xv[NB][8];
+#pragma unroll
+    for (int k = 0; k < N_IN; ++k)
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[k][b][u] = y[k * y_stride + static_cast<size_t>(r) * D + min(512 * b + lane + 64 * u, D - 1)];
+    float* xr = x + static_cast<size_t>(r) * D;
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) xv[b][u] = xr[min(512 * b + lane + 64 * u, D - 1)];
+    float inv[N_IN];
+#pragma unroll
+    for (int k = 0; k < N_IN; ++k) {
+        float ss = 0.f;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) ss += (512 * b + lane + 64 * u < D) ? v[k][b][u] * v[k][b][u] : 0.f;
+        inv[k] = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(D) + eps);
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        float g[N_IN][8];
+#pragma unroll
+        for (int k = 0; k < N_IN; ++k)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) g[k][u] = w[k * w_stride + min(512 * b + lane + 64 * u, D - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            float a = 0.f;
+#pragma unroll
+            for (int k = 0; k < N_IN; ++k) a += v[k][b][u] * inv[k] * g[k][u];
+            if (512 * b + lane + 64 * u < D) xr[512 * b + lane + 64 * u] = xv[b][u] + mult * a;
+        }
+    }
+}
+
 // The same two norms for rows whose parts are multiples of 4 and at most 2,048 long, 16-byte aligned: the part
 // lives in registers as float4, and every load is issued without a condition, from a clamped index, before the
 // first use (a load under a condition waits for all loads in flight, and a row of 768 then costs eight round trips).
@@ -284,6 +334,24 @@ int mllm_rmsnorm_add(float* y, const float* w, const float* scale, float mult, f
     if (vec && n >= 512) rmsnorm_add_vec_kernel<8><<<(n + 7) / 8, 512, 0, stream>>>(y, w, scale, mult, eps, x, n, D, clear);
     else if (vec) rmsnorm_add_vec_kernel<4><<<(n + 3) / 4, 256, 0, stream>>>(y, w, scale, mult, eps, x, n, D, clear);
     else rmsnorm_add_kernel<4><<<(n + 3) / 4, 256, 0, stream>>>(y, w, scale, mult, eps, x, n, D, clear);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+// -1: fewer than 2 or more than 4 inputs, or rows of more than 2,048 columns
+int mllm_rmsnorm_add_many(const float* y, size_t y_stride, const float* w, size_t w_stride, int n_in, float mult, float eps,
+                          float* x, int n, int D, hipStream_t stream) {
+    if (n <= 0 || D <= 0) return 0;
+    if (n_in < 2 || n_in > 4 || D > 2048) return -1;
+#define RAM(N_IN, NB)                                                                                                  \
+    do {                                                                                                               \
+        if (n >= 512) rmsnorm_add_many_kernel<8, N_IN, NB><<<(n + 7) / 8, 512, 0, stream>>>(y, y_stride, w, w_stride, mult, eps, x, n, D); \
+        else rmsnorm_add_many_kernel<4, N_IN, NB><<<(n + 3) / 4, 256, 0, stream>>>(y, y_stride, w, w_stride, mult, eps, x, n, D); \
+    } while (0)
+#define RAM_NB(N_IN) do { if (D <= 512) RAM(N_IN, 1); else if (D <= 1024) RAM(N_IN, 2); else RAM(N_IN, 4); } while (0)
+    if (n_in == 2) RAM_NB(2); else if (n_in == 3) RAM_NB(3); else RAM_NB(4);
+#undef RAM_NB
+#undef RAM
     MLLM_LAUNCH_CHECK();
     return 0;
 }

@@ -67,6 +67,71 @@ __global__ void conv_residual_kernel(const float* __restrict__ in, int ld, int C
     out[static_cast<size_t>(t) * ldo + ch] = from_float<OutT>(own + acc);
 }
 
+// A step in which every sequence brings one token: h = x / sqrt(mean(x^2) + eps) * wn and out = h + conv(h) in one
+// kernel, one wavefront per token. The earlier inputs of the convolution are the slot's carried rows, which move up
+// by one behind the read; h becomes the newest.
+// NB blocks of 512 columns: the row of x stays in registers between the statistics and the convolution. All loads of a
+// block are issued together, without conditions, from clamped (always valid) places, and masked where they are used
+// (a load under a condition, or in a loop of unknown length, is waited for before the next is asked for); TAPS is a
+// constant for that reason.
+template <typename OutT, int WAVES, int TAPS, int NB>
+__global__ void __launch_bounds__(64 * WAVES)
+rmsnorm_conv_single_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ wn, float eps, int C,
+                           const float* __restrict__ wc, const int* __restrict__ state_slots, float* __restrict__ state,
+                           size_t slot_floats, OutT* __restrict__ out, int ldo, int T, int write) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
+    const int t = blockIdx.x * WAVES + wave;
+    if (t >= T) return;
+    const int slot = state_slots[t];
+    if (slot < 0) return;
+    const float* xr = x + static_cast<size_t>(t) * ldx;
+    float xv[NB][8];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) xv[b][u] = xr[min(512 * b + lane + 64 * u, C - 1)];
+    float ss = 0.f;
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) ss += (512 * b + lane + 64 * u < C) ? xv[b][u] * xv[b][u] : 0.f;
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(C) + eps);
+    float* carried = state + static_cast<size_t>(slot) * slot_floats;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        if (512 * b >= C) break;
+        int idx[8];
+        float g[8], w[TAPS][8], v[TAPS > 1 ? TAPS - 1 : 1][8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) idx[u] = min(512 * b + lane + 64 * u, C - 1);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) g[u] = wn[idx[u]];
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) w[j][u] = wc[static_cast<size_t>(idx[u]) * TAPS + j];
+#pragma unroll
+        for (int j = 0; j + 1 < TAPS; ++j)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[j][u] = carried[static_cast<size_t>(j) * C + idx[u]];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float h = xv[b][u] * inv * g[u];
+            float acc = w[TAPS - 1][u] * h;
+#pragma unroll
+            for (int j = 0; j + 1 < TAPS; ++j) acc += w[j][u] * v[j][u];
+            if (512 * b + lane + 64 * u < C) {
+                if (write) {
+#pragma unroll
+                    for (int j = 1; j + 1 < TAPS; ++j) carried[static_cast<size_t>(j - 1) * C + idx[u]] = v[j][u];
+                    if (TAPS > 1) carried[static_cast<size_t>(TAPS - 2) * C + idx[u]] = h;
+                }
+                out[static_cast<size_t>(t) * ldo + idx[u]] = from_float<OutT>(h + acc);
+            }
+        }
+    }
+}
+
 // The slot's carried rows after the portion: its last taps - 1 inputs, older ones shifted out; a portion
 // shorter than that keeps the newest of the old rows. One thread per (sequence, channel); taps - 1 <= 15.
 __global__ void conv_carry_kernel(const float* __restrict__ proj, int ld, int col0, int C, int taps,
@@ -455,6 +520,33 @@ int mllm_conv_residual(const float* in, int ld, int C, const float* w, int taps,
                                                                                     slot_floats, B);
         MLLM_LAUNCH_CHECK();
     }
+    return 0;
+}
+
+// out = h + conv(h), h = rmsnorm(x) * wn, for a step of T sequences of one token each (token t is sequence t).
+// -1: taps outside 1..16; -2: more than 8 taps or rows of more than 2,048 columns (nothing is launched).
+int mllm_rmsnorm_conv_single(const float* x, int ldx, const float* wn, float eps, int C, const float* wc, int taps,
+                             const int* state_slots, float* state, size_t slot_floats, void* out, int ldo, int out_dtype, int T,
+                             int write, hipStream_t stream) {
+    if (T <= 0 || C <= 0) return 0;
+    if (taps < 1 || taps > 16) return -1;
+    if (taps > 8 || C > 2048) return -2;           // sizes this kernel is not made for: norm and convolution apart
+#define RCS(TYPE, TAPS, NB)                                                                                            \
+    rmsnorm_conv_single_kernel<TYPE, 4, TAPS, NB><<<(T + 3) / 4, 256, 0, stream>>>(x, ldx, wn, eps, C, wc, state_slots, state, \
+                                                                                  slot_floats, static_cast<TYPE*>(out), ldo, T, write)
+#define RCS_NB(TYPE, TAPS)                                                                                             \
+    do { if (C <= 512) RCS(TYPE, TAPS, 1); else if (C <= 1024) RCS(TYPE, TAPS, 2); else RCS(TYPE, TAPS, 4); } while (0)
+#define RCS_TAPS(TYPE)                                                                                                 \
+    switch (taps) {                                                                                                    \
+        case 1: RCS_NB(TYPE, 1); break; case 2: RCS_NB(TYPE, 2); break; case 3: RCS_NB(TYPE, 3); break;                \
+        case 4: RCS_NB(TYPE, 4); break; case 5: RCS_NB(TYPE, 5); break; case 6: RCS_NB(TYPE, 6); break;                \
+        case 7: RCS_NB(TYPE, 7); break; default: RCS_NB(TYPE, 8); break;                                               \
+    }
+    if (out_dtype == MLLM_F32) { RCS_TAPS(float) } else { RCS_TAPS(bf16_t) }
+#undef RCS_TAPS
+#undef RCS_NB
+#undef RCS
+    MLLM_LAUNCH_CHECK();
     return 0;
 }
 
