@@ -90,6 +90,86 @@ qk_prepare_kernel(const float* __restrict__ proj, int ld, int q_col, int k_col, 
     }
 }
 
+// The same for steps of few rows (decoding), one wavefront per (token, head): queries, then keys. A head of the
+// whole-row norm adds up the whole row itself (a few loads a lane) instead of waiting for the other heads. A lane has
+// up to 4 columns of its head (d <= 256); rotation partners meet through the wavefront's LDS.
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_prepare_heads_kernel(const float* __restrict__ proj, int ld, int q_col, int k_col, int v_col, int n_tokens, int H, int G, int d,
+                        int dv, int norm_mode, const float* __restrict__ wq, const float* __restrict__ wk, float eps, int rot_dims,
+                        double rot_base, const int* __restrict__ positions, const int* __restrict__ slots, T* __restrict__ q_out,
+                        int ldq, T* __restrict__ k_pages, T* __restrict__ v_pages) {
+    __shared__ float normed_s[4][256];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), lane = threadIdx.x % 64;
+    const int pair = blockIdx.x * 4 + wave;
+    if (pair >= n_tokens * (H + G)) return;           // the whole wavefront leaves; no workgroup barrier below
+    const int t = pair / (H + G), hh = pair % (H + G);
+    const bool is_k = hh >= H;
+    const int h = is_k ? hh - H : hh, n_row = (is_k ? G : H) * d;
+    const float* row = proj + static_cast<size_t>(t) * ld + (is_k ? k_col : q_col);
+    const float* wn = is_k ? wk : wq;
+    float raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) raw[u] = row[h * d + min(lane + 64 * u, d - 1)];
+    float inv = 1.f;
+    if (norm_mode == NORM_HEAD) {
+        float ss = 0.f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) ss += (lane + 64 * u < d) ? raw[u] * raw[u] : 0.f;
+        inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(d) + eps);
+    } else if (norm_mode == NORM_ROW) {
+        float ss = 0.f;
+        for (int base = 0; base < n_row; base += 512) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = row[min(base + lane + 64 * u, n_row - 1)];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) ss += (base + lane + 64 * u < n_row) ? v[u] * v[u] : 0.f;
+        }
+        inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(n_row) + eps);
+    }
+    const int half = rot_dims / 2;
+    float* mine = normed_s[threadIdx.x / 64];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int i = lane + 64 * u;
+        if (i < d) {
+            float g = 1.f;
+            if (norm_mode == NORM_HEAD) g = wn[i];
+            if (norm_mode == NORM_ROW) g = wn[h * d + i];
+            mine[i] = norm_mode == NORM_NONE ? raw[u] : raw[u] * inv * g;
+        }
+    }
+    wave_lds_sync();
+    const int slot = slots[t];
+    const double pos = static_cast<double>(positions[t]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int i = lane + 64 * u;
+        if (i >= d) continue;
+        float val = mine[i];
+        if (i < rot_dims) {
+            // the angle in double, rounded once
+            const int pi = i < half ? i : i - half;
+            const double a = pos * pow(rot_base, -2.0 * pi / rot_dims);
+            const float c = static_cast<float>(cos(a)), sn = static_cast<float>(sin(a));
+            val = i < half ? val * c - mine[i + half] * sn : val * c + mine[i - half] * sn;
+        }
+        if (!is_k) q_out[static_cast<size_t>(t) * ldq + h * d + i] = from_float<T>(val);
+        else if (slot >= 0) k_pages[static_cast<size_t>(slot) * G * d + h * d + i] = from_float<T>(val);
+    }
+    if (!is_k || slot < 0) return;
+    T* vp = v_pages + static_cast<size_t>(slot) * G * dv + h * dv;
+    if (v_col < 0) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (lane + 64 * u < d) vp[lane + 64 * u] = from_float<T>(raw[u]);
+    } else {
+        const float* vr = proj + static_cast<size_t>(t) * ld + v_col + h * dv;
+        for (int i = lane; i < dv; i += 64) vp[i] = from_float<T>(vr[i]);
+    }
+}
+
 struct ScoreShape {
     float scale, softcap;            // softcap <= 0: none
     int window, chunk;               // at most one of them > 0
@@ -230,6 +310,20 @@ int mllm_qk_prepare(const float* proj, int ld, int q_col, int k_col, int v_col, 
     if (H < 1 || G < 1 || d < 1 || dv < 1 || rot_dims < 0 || rot_dims % 2 != 0 || rot_dims > d || rot_dims / 2 > 256) return -1;
     if (v_col < 0 && dv != d) return -1;
     if (norm_mode != NORM_NONE && (wq == nullptr || wk == nullptr)) return -1;
+    if (T <= 64 && d <= 256) {
+        // few rows: one wavefront per (token, head) instead of one workgroup per token
+        const int blocks = (T * (H + G) + 3) / 4;
+        if (dtype == MLLM_F32)
+            qk_prepare_heads_kernel<float><<<blocks, 256, 0, stream>>>(proj, ld, q_col, k_col, v_col, T, H, G, d, dv, norm_mode, wq, wk, eps,
+                                                                       rot_dims, rot_base, positions, slots, static_cast<float*>(q_out), ldq,
+                                                                       static_cast<float*>(k_pages), static_cast<float*>(v_pages));
+        else
+            qk_prepare_heads_kernel<bf16_t><<<blocks, 256, 0, stream>>>(proj, ld, q_col, k_col, v_col, T, H, G, d, dv, norm_mode, wq, wk, eps,
+                                                                        rot_dims, rot_base, positions, slots, static_cast<bf16_t*>(q_out), ldq,
+                                                                        static_cast<bf16_t*>(k_pages), static_cast<bf16_t*>(v_pages));
+        MLLM_LAUNCH_CHECK();
+        return 0;
+    }
     const size_t smem = (static_cast<size_t>(H + G) * d + rot_dims + (H + G) + 2) * sizeof(float);
     if (smem > 60 * 1024) return -1;
     if (dtype == MLLM_F32)
