@@ -46,6 +46,7 @@ def test_native_readers_survive_damaged_files_under_sanitizers(tmp_path):
     build = subprocess.run([cxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
                             "-static-libasan", "-static-libubsan", "-x", "c++", "-D__HIP_PLATFORM_AMD__",
                             "-I/opt/rocm/include", "-I" + eng, "-I" + os.path.join(ROOT, "mini_llm_amd", "csrc", "runtime"),
+                            "-I" + os.path.join(ROOT, "mini_llm_amd", "csrc", "kernels"),
                             os.path.join(ROOT, "tests", "native", "loader_fuzz.cc"), os.path.join(eng, "json.cc"),
                             os.path.join(eng, "weights.cc"), "-o", exe, "-L/opt/rocm/lib", "-lamdhip64",
                             "-Wl,-rpath,/opt/rocm/lib", "-lpthread"], capture_output=True, text=True, timeout=600)
