@@ -246,6 +246,13 @@ public:
     virtual ~Mixer() = default;
     virtual void forward(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write,
                          Arena& arena, hipStream_t s) const = 0;
+    // The same, but x is SET to the mixer's output (x need not hold anything before). A mixer whose last product can
+    // store instead of add overrides this; otherwise x is cleared first.
+    virtual void forward_set(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write,
+                             Arena& arena, hipStream_t s) const {
+        fill_zero(x, s);
+        forward(h, step, cache, x, write, arena, s);
+    }
     virtual size_t workspace_bytes(int tokens) const = 0;
     virtual CacheNeed cache_need() const = 0;
     // Scratch that the mixer's kernels need on stream `s` for steps of up to max_seqs sequences: taken

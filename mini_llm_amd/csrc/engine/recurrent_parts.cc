@@ -1,5 +1,7 @@
 // The gated linear recurrence (HGRN2) as a mixer, mixers that run side by side, the gated feed-forward with
 // biases, the token table with a norm behind it, and the stream step that mixes the embedding's output back in.
+#include <algorithm>
+
 #include "parts.h"
 
 namespace minillm {
@@ -38,6 +40,14 @@ public:
     }
     void forward(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write, Arena& arena,
                  hipStream_t s) const override {
+        run(h, step, cache, x, write, arena, s, ADD_RESIDUAL);
+    }
+    void forward_set(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write, Arena& arena,
+                     hipStream_t s) const override {
+        run(h, step, cache, x, write, arena, s, STORE_F32);
+    }
+    void run(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write, Arena& arena,
+             hipStream_t s, int out_epilogue) const {
         if (!cache.has_state() || cache.state_bytes < state_floats_ * 4) fail("hgrn2 needs a state of %zu floats per request", state_floats_);
         const int T = step.n_tokens, N = in_.out_features(), ld = (N + 3) / 4 * 4, inner = H_ * dv_;
         Tensor2 proj(arena.take(static_cast<size_t>(T) * ld * 4), F32, T, N, ld);
@@ -57,12 +67,14 @@ public:
         StageTimes::get().mark("scan", s);
         Tensor2 normed = arena.tensor(dtype_, T, inner);
         rmsnorm(y, norm_, eps_, H_, nullptr, normed, nullptr, s, parts, static_cast<size_t>(T) * inner);
-        out_(normed, x, ADD_RESIDUAL, nullptr, s);
+        out_(normed, x, out_epilogue, nullptr, s);
         StageTimes::get().mark("out_proj", s);
     }
     size_t workspace_bytes(int tokens) const override {
         return static_cast<size_t>(tokens) * ((in_.out_features() + 4) * 4 + hgrn2_parts(d_) * H_ * dv_ * 4 + (H_ * dv_ + in_.in_features()) * dtype_size(dtype_)) +
-               hgrn2_workspace_floats(tokens, 1, H_, d_, dv_) * 4 + 8192;
+               // (every sequence of a step adds at most one chunk that is not full; a step holds at most as many
+               // sequences as tokens)
+               hgrn2_workspace_floats(tokens, std::min(tokens, 256), H_, d_, dv_) * 4 + 8192;
     }
     CacheNeed cache_need() const override {
         CacheNeed n;
@@ -87,8 +99,8 @@ private:
 };
 
 // Mixers side by side on the same input: x += (1 / n) sum_k rmsnorm(mixer_k(h)) * weight_k, every mixer's output
-// RMS-normed over the stream's width with a weight of its own before the mean is taken. Each mixer adds into a
-// cleared fp32 buffer of the stream's shape. At most one of them may keep pages; their states lie one behind the
+// RMS-normed over the stream's width with a weight of its own before the mean is taken. Each mixer sets an fp32
+// buffer of the stream's shape (Mixer::forward_set). At most one of them may keep pages; their states lie one behind the
 // other in the layer's state slot. Parameters: size, eps; mixers; tensors norm0, norm1, ... and optionally
 // norms (the same weights one behind the other: the norms and the mean then run in one kernel).
 class ParallelMixers final : public Mixer {
@@ -115,8 +127,7 @@ public:
                  hipStream_t s) const override {
         const int n = static_cast<int>(mixers_.size());
         if (x.cols != size_) fail("parallel mixers of width %d were handed a stream of %lld", size_, (long long)x.cols);
-        Tensor2 all = arena.tensor(F32, x.rows * n, x.cols);
-        fill_zero(all, s);
+        Tensor2 all = arena.tensor(F32, x.rows * n, x.cols);          // (every mixer sets its own share)
         size_t state_at = 0;
         for (int k = 0; k < n; ++k) {
             const CacheNeed need = mixers_[k]->cache_need();
@@ -134,7 +145,7 @@ public:
                 state_at += (need.state_bytes + 15) / 16 * 16;
             }
             const size_t mark = arena.mark();
-            mixers_[k]->forward(h, step, mine, all.row_range(x.rows * k, x.rows), write, arena, s);
+            mixers_[k]->forward_set(h, step, mine, all.row_range(x.rows * k, x.rows), write, arena, s);
             arena.release(mark);
         }
         if (joined_norms_ != nullptr && n <= 4 && x.cols <= 2048) rmsnorm_add_many(all, joined_norms_, n, 1.0f / n, eps_, x, s);

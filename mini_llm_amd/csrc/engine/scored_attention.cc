@@ -64,6 +64,14 @@ public:
     }
     void forward(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write, Arena& arena,
                  hipStream_t s) const override {
+        run(h, step, cache, x, write, arena, s, ADD_RESIDUAL);
+    }
+    void forward_set(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write, Arena& arena,
+                     hipStream_t s) const override {
+        run(h, step, cache, x, write, arena, s, STORE_F32);
+    }
+    void run(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write, Arena& arena,
+             hipStream_t s, int out_epilogue) const {
         if (!cache.has_pages()) fail("scored_attention needs a cache of pages");
         if (!write) fail("scored_attention writes its own keys and values: it cannot read another call's cache");
         const int T = step.n_tokens, g = cache.group, N = in_.out_features(), ld = (N + 3) / 4 * 4;
@@ -79,7 +87,7 @@ public:
         Tensor2 o = arena.tensor(dtype_, T, sh_.n_heads * sh_.value_dim);
         scored_attention(q, cache.k_pages, cache.v_pages, st, sh_, gated_ ? &proj : nullptr, gate_col_, o, s);
         StageTimes::get().mark("attention", s);
-        out_(o, x, ADD_RESIDUAL, nullptr, s);
+        out_(o, x, out_epilogue, nullptr, s);
         StageTimes::get().mark("out_proj", s);
     }
     size_t workspace_bytes(int tokens) const override {

@@ -191,7 +191,7 @@ __device__ __forceinline__ float shaped_score(float dot, const ScoreShape& sh, f
 }
 
 #define SA_WAVES 4
-#define SA_MAX_ACC 4   // value rows of up to 64 * SA_MAX_ACC columns
+#define SA_MAX_ACC 8   // value rows of up to 64 * SA_MAX_ACC columns
 
 // One wavefront per (query token, head): 64 keys a round, one key per lane for the scores, then one value
 // column (or a few) per lane for the sum. Any sizes; serves prompt portions and single tokens alike.
@@ -219,7 +219,9 @@ scored_attention_rows(const T* __restrict__ q, int ldq, const T* __restrict__ k_
     const int kd = G * d, vd = G * dv;
     const bool vec = d % 8 == 0 && (kd * sizeof(T)) % 16 == 0 && (reinterpret_cast<uintptr_t>(k_pages) & 15) == 0;
     float m = -INFINITY, l = 0.f;
-    float acc[SA_MAX_ACC] = {0.f, 0.f, 0.f, 0.f};
+    float acc[SA_MAX_ACC];
+#pragma unroll
+    for (int a = 0; a < SA_MAX_ACC; ++a) acc[a] = 0.f;
     for (int j0 = lo; j0 <= p; j0 += 64) {
         const int j = j0 + lane;
         const bool valid = j <= p;
