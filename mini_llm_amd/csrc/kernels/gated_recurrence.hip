@@ -26,7 +26,7 @@ __device__ __forceinline__ float gr_sigmoid(float v) { return 1.f / (1.f + expf(
 // MODE 2: every chunk again, from the state it starts from, results to y.
 // The sums are those of the token-by-token recurrence in another order.
 // Workspace per chunk and head: [d * dv] the chunk's state, then [d] the product of its gates.
-#define GR_CHUNK 64
+#define GR_CHUNK 32
 
 template <int MODE>
 __global__ void __launch_bounds__(64)
