@@ -110,3 +110,19 @@ def test_plain_prompt_equals_token_by_token_through_the_convolution(tmp_path):
     full = pr.forward(cfg, w, toks)
     for n in (1, 5, 12):
         assert torch.allclose(pr.forward(cfg, w, toks[:n]), full[:n], atol=1e-10)
+
+
+@pytest.mark.parametrize("size", ["gpt2-small", "gpt2-medium", "gpt2-xl"])
+def test_the_benchmark_configuration_is_a_model(size):
+    """bench.py --design rekirax: its configuration at every size is one the architecture takes, with as many layer
+    runs as the GPT-2 configuration of that size has layers."""
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+    cfg = bench.rekirax_config(0, size)
+    d = describe_config(cfg)
+    assert d["architecture"] == "Rekirax"
+    assert len(pr.layer_runs(cfg)) == bench.SIZES[size][0] == cfg["n_layer"]
+    shapes = {t["name"]: t["shape"] for t in d["tensors"]}
+    assert shapes["embed"][1] == bench.SIZES[size][1] and "loop.in" in shapes

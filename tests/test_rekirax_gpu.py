@@ -138,6 +138,18 @@ def test_far_keys_among_hundreds_with_peaked_scores(dirs, page):
                                tol=rc.TOL_PEAKED)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_prompt_of_a_thousand_tokens(dirs, dtype):
+    """One prompt of 1,100 tokens whole, in portions of hundreds and of two tokens, and with its last tokens one by
+    one: many key tiles, many chunks of the scan, block tables of dozens of pages."""
+    cfg, d = rc.SHARED_KERNELS, dirs("SHARED_KERNELS")
+    reqs = rc.requests(cfg["vocab"], [1100], seed=81)
+    for label, steps in (("whole", ru.trace_whole(reqs)), ("chunks", ru.trace_chunks(reqs, seed=8, sizes=(300, 2, 129, 64, 401))),
+                         ("decode", ru.trace_decode_tail(reqs, tail=25))):
+        runner = _runner(d, dtype, n_pages=ru.peak_tokens(steps) // 16, page=16)
+        rc.check_against_plain(d, reqs, steps, ru.run_in_process(runner, steps), dtype, cfg["vocab"], f"long prompt {label}")
+
+
 @pytest.mark.parametrize("what", ["window", "chunk"])
 def test_peaked_scores_would_show_an_edge_one_key_off(dirs, what):
     """The tests above have teeth: the plain model with every window (or chunk) one key wider differs from the
