@@ -99,6 +99,46 @@ rmsnorm_add_kernel(float* __restrict__ y, const float* __restrict__ w, const flo
     }
 }
 
+// Many short groups (heads of a recurrence: 16 to 128 columns each): LANES = columns / 4 lanes take one (row, group)
+// pair, a wavefront 64 / LANES of them, so that every lane holds four columns whatever the group's size (one wavefront
+// per pair leaves 48 of 64 lanes idle at 64 columns). Up to four shares are added in the order of their index; no
+// gate, no row selection. All loads without conditions, from clamped places.
+template <typename OutT, int LANES>
+__global__ void __launch_bounds__(256)
+rmsnorm_small_groups_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ w, OutT* __restrict__ y, int ldy,
+                            long long pairs, int groups, float eps, int parts, size_t part_stride) {
+    constexpr int PER_WAVE = 64 / LANES, DG = 4 * LANES;
+    const int lane = threadIdx.x % MLLM_WAVE, sub = lane % LANES;
+    const long long wave = static_cast<long long>(blockIdx.x) * 4 + threadIdx.x / MLLM_WAVE;
+    const long long mine = wave * PER_WAVE + lane / LANES;
+    const bool valid = mine < pairs;
+    const long long pair = valid ? mine : pairs - 1;
+    const long long r = pair / groups;
+    const int g = static_cast<int>(pair % groups);
+    const float* xr = x + static_cast<size_t>(r) * ldx + g * DG + 4 * sub;
+    float4 v = *reinterpret_cast<const float4*>(xr);
+    float4 sh[3];
+#pragma unroll
+    for (int part = 1; part < 4; ++part) sh[part - 1] = *reinterpret_cast<const float4*>(xr + min(part, parts - 1) * part_stride);
+    const float4 ww = *reinterpret_cast<const float4*>(w + g * DG + 4 * sub);
+#pragma unroll
+    for (int part = 1; part < 4; ++part)
+        if (part < parts) { v.x += sh[part - 1].x; v.y += sh[part - 1].y; v.z += sh[part - 1].z; v.w += sh[part - 1].w; }
+    const float ss = group_sum<LANES>((v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w));
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(DG) + eps);
+    if (!valid) return;
+    OutT* yr = y + static_cast<size_t>(r) * ldy + g * DG + 4 * sub;
+    const float o0 = v.x * inv * ww.x, o1 = v.y * inv * ww.y, o2 = v.z * inv * ww.z, o3 = v.w * inv * ww.w;
+    if (sizeof(OutT) == 2) {
+        uint2 pk;
+        pk.x = pack_bf16x2(o0, o1);
+        pk.y = pack_bf16x2(o2, o3);
+        *reinterpret_cast<uint2*>(yr) = pk;
+    } else {
+        *reinterpret_cast<float4*>(yr) = make_float4(o0, o1, o2, o3);
+    }
+}
+
 // x[r, i] += mult * sum_k y_k[r, i] / sqrt(mean(y_k[r]^2) + eps) * w_k[i] for n inputs of x's shape that lie
 // y_stride floats apart (weights w_stride apart), added in the order of k; one wavefront per row.
 // N_IN inputs, NB blocks of 512 columns: every input row stays in registers between its statistics and the sum; loads
@@ -311,7 +351,18 @@ int mllm_rmsnorm(const float* x, int ldx, const int* rows, const float* w, const
 #define RMS_SHARES(TYPE)                                                                                                \
     rmsnorm_vec_kernel<TYPE, 4, true><<<static_cast<int>((pairs + 3) / 4), 256, 0, stream>>>(                           \
         x, ldx, rows, w, gate, ldg, static_cast<TYPE*>(y), ldy, n, D, groups, eps, parts, part_stride)
-    if (vec && parts > 1) {
+    if (vec && groups > 1 && rows == nullptr && gate == nullptr && (Dg == 16 || Dg == 32 || Dg == 64 || Dg == 128)) {
+        // many short groups: several of them a wavefront
+        const int per_wg = 4 * (64 / (Dg / 4));
+        const int blocks = static_cast<int>((pairs + per_wg - 1) / per_wg);
+#define RSG(TYPE, LANES)                                                                                              \
+    rmsnorm_small_groups_kernel<TYPE, LANES><<<blocks, 256, 0, stream>>>(x, ldx, w, static_cast<TYPE*>(y), ldy, pairs, groups, eps, parts, \
+                                                                        part_stride)
+#define RSG_T(TYPE) do { if (Dg == 16) RSG(TYPE, 4); else if (Dg == 32) RSG(TYPE, 8); else if (Dg == 64) RSG(TYPE, 16); else RSG(TYPE, 32); } while (0)
+        if (out_dtype == MLLM_F32) RSG_T(float); else RSG_T(bf16_t);
+#undef RSG_T
+#undef RSG
+    } else if (vec && parts > 1) {
         if (out_dtype == MLLM_F32) RMS_SHARES(float); else RMS_SHARES(bf16_t);
     } else if (vec) {
         if (out_dtype == MLLM_F32) { if (pairs >= 512) RMS(rmsnorm_vec_kernel, float, 8); else RMS(rmsnorm_vec_kernel, float, 4); }
